@@ -22,24 +22,12 @@
 // The state is kept transposed, [slot][head][value channel][key channel], so that a lane's rows are contiguous.
 #include "common.h"
 #include "fmsamd.h"
+#include "short_conv.h"
 
-#define DELTA_MAX_TAPS 8
+#define DELTA_MAX_TAPS CONV_MAX_TAPS
 
 __device__ __forceinline__ float softplus_f32(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 __device__ __forceinline__ float sigmoid_f32(float z) { return 1.f / (1.f + expf(-z)); }
-
-// How many tokens of its sequence come before token t in the step, up to taps - 1 (all that a convolution of `taps`
-// taps needs to know).  The candidates are loaded together, not one after another.
-__device__ __forceinline__ int tokens_before(const int* __restrict__ seq_of_token, int t, int seq, int taps) {
-  int prev[DELTA_MAX_TAPS - 1];
-#pragma unroll
-  for (int d = 1; d < DELTA_MAX_TAPS; ++d) prev[d - 1] = (d < taps && t - d >= 0) ? seq_of_token[t - d] : -2;
-  int have = 0;
-#pragma unroll
-  for (int d = 1; d < DELTA_MAX_TAPS; ++d)
-    if (have == d - 1 && prev[d - 1] == seq) have = d;
-  return have;
-}
 
 // Blocks of 1024 threads for steps of few tokens (a decode step has a block per token and nothing else to hide a
 // load's latency behind: the fewer passes a thread makes, the fewer round trips to memory follow one another).
@@ -108,31 +96,6 @@ __global__ void __launch_bounds__(1024)
   for (int i = threadIdx.x; i < H * per_head; i += blockDim.x) {
     const float z = a[(size_t)t * lda + col_a + i] + dt_bias[i];
     decay[(size_t)t * H * per_head + i] = expf(-expf(a_log[i / per_head]) * softplus_f32(z));
-  }
-}
-
-// Runs after delta_prepare of the same step (which reads the old state).  The block of a sequence's last token of the
-// step writes; new entry s is either a row of the step or an old entry above s.
-__global__ void __launch_bounds__(1024)
-    conv_state_kernel(const float* __restrict__ proj, long ld, int taps, float* __restrict__ conv_state,
-                      const int* __restrict__ seq_of_token, const int* __restrict__ slot_ids, int n_tokens, int C) {
-  const int t = blockIdx.x;
-  const int seq = seq_of_token[t];
-  if (seq < 0) return;
-  if (t + 1 < n_tokens && seq_of_token[t + 1] == seq) return;  // not the sequence's last token of the step
-  const int have = tokens_before(seq_of_token, t, seq, taps);
-  float* state = conv_state + (size_t)slot_ids[seq] * (taps - 1) * C;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float fresh[DELTA_MAX_TAPS - 1];  // all of a channel's new entries are read before any is written
-#pragma unroll
-    for (int s = 0; s < DELTA_MAX_TAPS - 1; ++s) {
-      const int d = taps - 2 - s;  // new entry s is the input d tokens before the last one
-      fresh[s] = 0.f;
-      if (s < taps - 1) fresh[s] = d <= have ? proj[(size_t)(t - d) * ld + c] : state[(size_t)(taps - 1 + have - d) * C + c];
-    }
-#pragma unroll
-    for (int s = 0; s < DELTA_MAX_TAPS - 1; ++s)
-      if (s < taps - 1) state[(size_t)s * C + c] = fresh[s];
   }
 }
 

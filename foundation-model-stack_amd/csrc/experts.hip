@@ -81,6 +81,124 @@ extern "C" int fmsamd_moe_route(const float* logits, long ld, int n_tokens, int 
   return 0;
 }
 
+// The wave's largest value and where it is (ties: the lower index); every lane gets both.
+__device__ __forceinline__ void wave_argmax(float& best, int& at) {
+#pragma unroll
+  for (int off = WAVE / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off, WAVE);
+    const int oa = __shfl_xor(at, off, WAVE);
+    if (ov > best || (ov == best && oa < at)) best = ov, at = oa;
+  }
+}
+
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_wave_barrier();
+  __threadfence_block();
+}
+
+// Routing over groups of experts.  s = softmax over all n router outputs; an output is chosen by s + correction, but
+// weighted by s.  The outputs form `groups` equal runs of neighbours; a group's score is its largest choice score, and
+// only outputs of the `keep` best groups can be chosen (the others count as minus infinity).  The weights of the `top`
+// chosen are their s divided by their sum (+ 1e-20), times `scale`.  One wave per token; ties go to the lower index.
+__global__ void __launch_bounds__(256)
+    route_grouped_kernel(const float* __restrict__ logits, long ld, int n_tokens, int n, int top, const float* __restrict__ correction,
+                         int groups, int keep, float scale, int* __restrict__ ids, float* __restrict__ weights) {
+  extern __shared__ float lds[];  // 4 waves x (2 n + 2 groups + top)
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= n_tokens) return;
+  float* s = lds + (size_t)wave * (2 * n + 2 * groups + top);
+  float* choice = s + n;
+  float* gscore = choice + n;
+  float* kept = gscore + groups;
+  float* chosen = kept + groups;
+  float m = -INFINITY;
+  for (int e = lane; e < n; e += WAVE) {
+    const float z = logits[(size_t)t * ld + e];
+    s[e] = z;
+    m = fmaxf(m, z);
+  }
+  m = wave_max(m);
+  float sum = 0.f;
+  for (int e = lane; e < n; e += WAVE) {
+    const float p = expf(s[e] - m);
+    s[e] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  for (int e = lane; e < n; e += WAVE) {
+    const float p = s[e] / sum;
+    float c = p + (correction ? correction[e] : 0.f);
+    if (!(c >= -3.0e38f)) c = -3.0e38f;  // not a number (a padding row's logits): still a candidate, the last of all
+    s[e] = p;
+    choice[e] = c;
+  }
+  wave_lds_fence();
+  if (groups > 1) {
+    const int per = n / groups;
+    for (int g = lane; g < groups; g += WAVE) {
+      float best = -INFINITY;
+      for (int e = g * per; e < (g + 1) * per; ++e) best = fmaxf(best, choice[e]);
+      gscore[g] = best;
+      kept[g] = 0.f;
+    }
+    wave_lds_fence();
+    for (int j = 0; j < keep; ++j) {
+      float best = -INFINITY;
+      int at = 0x7fffffff;
+      for (int g = lane; g < groups; g += WAVE) {
+        const float v = gscore[g];
+        if (v > best || (v == best && g < at)) best = v, at = g;
+      }
+      wave_argmax(best, at);
+      if (lane == 0 && at < groups) kept[at] = 1.f, gscore[at] = -INFINITY;
+      wave_lds_fence();
+    }
+    for (int e = lane; e < n; e += WAVE)
+      if (kept[e / per] == 0.f) choice[e] = -INFINITY;
+    wave_lds_fence();
+  }
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < n; e += WAVE) {
+      const float v = choice[e];
+      if (v > best || (v == best && e < at)) best = v, at = e;
+    }
+    wave_argmax(best, at);
+    if (at >= n) at = 0;  // nothing left to choose from: the configuration allows fewer outputs than `top`
+    if (lane == 0) {
+      ids[(size_t)t * top + j] = at;
+      chosen[j] = s[at];
+      choice[at] = -INFINITY;
+    }
+    wave_lds_fence();
+  }
+  if (lane == 0) {
+    float total = 0.f;
+    for (int j = 0; j < top; ++j) total += chosen[j];
+    const float norm = scale / (total + 1e-20f);
+    for (int j = 0; j < top; ++j) weights[(size_t)t * top + j] = chosen[j] * norm;
+  }
+}
+
+extern "C" int fmsamd_moe_route_grouped(const float* logits, long ld, int n_tokens, int n_outputs, int top, const float* correction,
+                                        int groups, int keep, float scale, int* ids, float* weights, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && n_outputs > 0 && n_outputs <= ROUTE_MAX_EXPERTS && top > 0 && top <= n_outputs && top <= ROUTE_MAX_TOP,
+              "moe_route_grouped: %d outputs (at most %d), top %d (at most %d and the outputs)", n_outputs, ROUTE_MAX_EXPERTS, top,
+              ROUTE_MAX_TOP);
+  FMS_REQUIRE(ld >= n_outputs, "moe_route_grouped: rows of %ld for %d outputs", ld, n_outputs);
+  FMS_REQUIRE(groups >= 1 && n_outputs % groups == 0 && keep >= 1 && keep <= groups && (long)keep * (n_outputs / groups) >= top,
+              "moe_route_grouped: %d groups of %d outputs, %d kept, cannot give %d choices", groups, n_outputs / (groups > 0 ? groups : 1),
+              keep, top);
+  const size_t lds = 4 * (size_t)(2 * n_outputs + 2 * groups + top) * sizeof(float);
+  route_grouped_kernel<<<ceil_div(n_tokens, 4), 256, lds, stream>>>(logits, ld, n_tokens, n_outputs, top, correction, groups, keep, scale,
+                                                                    ids, weights);
+  FMS_LAUNCH_CHECK("moe_route_grouped");
+  return 0;
+}
+
 // --------------------------------------------------------------------------
 // group: order[0 .. n) = the pairs sorted by expert; tiles[i] = (expert, first row in order, rows), rows 0: no tile
 // --------------------------------------------------------------------------
@@ -155,6 +273,7 @@ struct ExpertArgs {
   int top, N, K;
   float limit, alpha, shift;
   const float* in_scale;  // gate_up: a factor per pair on the expert's input (applied to both float32 sums), or null
+  int act;  // gate_up without up weights (w2 null): hidden = act(x W1^T), one of FMS_ACT_*
 };
 
 __device__ __forceinline__ float pair_scale(const ExpertArgs& a, int sorted_row) {
@@ -167,6 +286,11 @@ __device__ __forceinline__ float clamp_gated(float g, float u, float limit, floa
   return g / (1.f + expf(-alpha * g)) * (u + shift);
 }
 
+// what an expert keeps between its two products: the clamped gated activation of (gate, up), or act(the one product)
+__device__ __forceinline__ float hidden_value(const ExpertArgs& a, bool gated, float g, float u) {
+  return gated ? clamp_gated(g, u, a.limit, a.alpha, a.shift) : fms_activate(g, a.act);
+}
+
 template <typename T>
 __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_fma_kernel(ExpertArgs a) {
   const int e = a.tiles[3 * blockIdx.x], start = a.tiles[3 * blockIdx.x + 1], rows = a.tiles[3 * blockIdx.x + 2];
@@ -176,9 +300,10 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_fma_kernel(Expert
   const T* wg = (const T*)a.w1 + (size_t)e * a.N * a.K;
   const T* wu = (const T*)a.w2 + (size_t)e * a.N * a.K;
   auto a_row = [&](int m) { return m < rows ? x + (size_t)(a.order[start + m] / a.top) * a.ldx : (const T*)nullptr; };
-  float g[4], u[4];
+  const bool gated = a.w2 != nullptr;
+  float g[4], u[4] = {0.f, 0.f, 0.f, 0.f};
   tile_product_fma<T>(a_row, [&](int n) { return n0 + n < a.N ? wg + (size_t)(n0 + n) * a.K : (const T*)nullptr; }, a.K, g);
-  tile_product_fma<T>(a_row, [&](int n) { return n0 + n < a.N ? wu + (size_t)(n0 + n) * a.K : (const T*)nullptr; }, a.K, u);
+  if (gated) tile_product_fma<T>(a_row, [&](int n) { return n0 + n < a.N ? wu + (size_t)(n0 + n) * a.K : (const T*)nullptr; }, a.K, u);
   const int n = n0 + threadIdx.x % 64;
   if (n >= a.N) return;
 #pragma unroll
@@ -186,7 +311,7 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_fma_kernel(Expert
     const int m = (threadIdx.x / 64) * 4 + i;
     if (m < rows) {
       const float sc = pair_scale(a, start + m);
-      ((T*)a.y)[(size_t)(start + m) * a.N + n] = from_f32<T>(clamp_gated(g[i] * sc, u[i] * sc, a.limit, a.alpha, a.shift));
+      ((T*)a.y)[(size_t)(start + m) * a.N + n] = from_f32<T>(hidden_value(a, gated, g[i] * sc, u[i] * sc));
     }
   }
 }
@@ -218,9 +343,12 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_mfma_kernel(Exper
   const bf16* wg = (const bf16*)a.w1 + (size_t)e * a.N * a.K;
   const bf16* wu = (const bf16*)a.w2 + (size_t)e * a.N * a.K;
   auto a_row = [&](int m) { return m < rows ? x + (size_t)(a.order[start + m] / a.top) * a.ldx : (const bf16*)nullptr; };
+  const bool gated = a.w2 != nullptr;
   f32x4 g[TILE_MFMA_WAVE_TILES], u[TILE_MFMA_WAVE_TILES];
+#pragma unroll
+  for (int tl = 0; tl < TILE_MFMA_WAVE_TILES; ++tl) u[tl] = f32x4{0.f, 0.f, 0.f, 0.f};
   tile_product_mfma(a_row, [&](int n) { return n0 + n < a.N ? wg + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, g);
-  tile_product_mfma(a_row, [&](int n) { return n0 + n < a.N ? wu + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, u);
+  if (gated) tile_product_mfma(a_row, [&](int n) { return n0 + n < a.N ? wu + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, u);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -230,7 +358,7 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_mfma_kernel(Exper
 #pragma unroll
     for (int tl = 0; tl < TILE_MFMA_WAVE_TILES; ++tl) {
       const int n = n0 + wave * (16 * TILE_MFMA_WAVE_TILES) + tl * 16 + (lane & 15);
-      if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)clamp_gated(g[tl][i] * sc, u[tl][i] * sc, a.limit, a.alpha, a.shift);
+      if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)hidden_value(a, gated, g[tl][i] * sc, u[tl][i] * sc);
     }
   }
 }
@@ -267,9 +395,14 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_wide_kernel(Exper
   const bf16* wg = (const bf16*)a.w1 + (size_t)e * a.N * a.K;
   const bf16* wu = (const bf16*)a.w2 + (size_t)e * a.N * a.K;
   auto a_row = [&](int m) { return m < rows ? x + (size_t)(a.order[start + m] / a.top) * a.ldx : (const bf16*)nullptr; };
+  const bool gated = a.w2 != nullptr;
   f32x4 g[2][4], u[2][4];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) u[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
   tile_product_mfma_wide(a_row, [&](int n) { return n0 + n < a.N ? wg + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, g);
-  tile_product_mfma_wide(a_row, [&](int n) { return n0 + n < a.N ? wu + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, u);
+  if (gated) tile_product_mfma_wide(a_row, [&](int n) { return n0 + n < a.N ? wu + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, u);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
   for (int mt = 0; mt < 2; ++mt) {
@@ -281,7 +414,7 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_wide_kernel(Exper
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt) {
         const int n = n0 + (wave & 1) * 64 + nt * 16 + (lane & 15);
-        if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)clamp_gated(g[mt][nt][i] * sc, u[mt][nt][i] * sc, a.limit, a.alpha, a.shift);
+        if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)hidden_value(a, gated, g[mt][nt][i] * sc, u[mt][nt][i] * sc);
       }
     }
   }
@@ -317,13 +450,14 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_down_wide_kernel(ExpertAr
 // tile_rows: what fmsamd_moe_tile_rows said when the tiles were made
 extern "C" int fmsamd_moe_experts(int stage, const void* x, long ldx, const void* w1, const void* w2, void* y, int dtype,
                                   const int* order, const int* tiles, int max_tiles, int tile_rows, int top, int N, int K,
-                                  float limit, float alpha, float shift, const float* in_scale, hipStream_t stream) {
+                                  float limit, float alpha, float shift, const float* in_scale, int act, hipStream_t stream) {
   if (max_tiles == 0) return 0;
+  FMS_REQUIRE(act >= 0 && act <= FMS_ACT_LAST, "moe_experts: unknown activation %d", act);
   FMS_REQUIRE(stage == 0 || stage == 1, "moe_experts: stage %d", stage);
   FMS_REQUIRE(tile_rows == TILE_ROWS || tile_rows == TILE_WIDE_ROWS, "moe_experts: tiles of %d rows", tile_rows);
   FMS_REQUIRE(max_tiles > 0 && top > 0 && N > 0 && K > 0 && ldx >= K, "moe_experts: bad sizes tiles=%d top=%d N=%d K=%d ldx=%ld", max_tiles,
               top, N, K, ldx);
-  ExpertArgs a{x, ldx, w1, w2, y, order, tiles, top, N, K, limit, alpha, shift, stage == 0 ? in_scale : nullptr};
+  ExpertArgs a{x, ldx, w1, w2, y, order, tiles, top, N, K, limit, alpha, shift, stage == 0 ? in_scale : nullptr, act};
   const bool mfma = dtype == FMS_BF16 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w1 % 16) == 0 &&
                     (w2 == nullptr || ((uintptr_t)w2 % 16) == 0);
   const dim3 grid(max_tiles, ceil_div(N, mfma ? TILE_MFMA_COLS : TILE_FMA_COLS));
@@ -357,12 +491,18 @@ extern "C" int fmsamd_moe_experts(int stage, const void* x, long ldx, const void
 template <typename T>
 __global__ void __launch_bounds__(256)
     combine_kernel(const float* __restrict__ y, const float* __restrict__ weights, int top, const T* __restrict__ shared,
-                   const float* __restrict__ shared_gate, long ldg, T* __restrict__ out, int width) {
+                   const float* __restrict__ shared_gate, long ldg, T* __restrict__ out, int width, const int* __restrict__ ids,
+                   int n_experts, const T* __restrict__ x_in, long ldx) {
   const int t = blockIdx.x;
   const float sg = shared ? (shared_gate ? 1.f / (1.f + expf(-shared_gate[(size_t)t * ldg])) : 1.f) : 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float v = 0.f;
-    for (int j = 0; j < top; ++j) v = fmaf(weights ? weights[(size_t)t * top + j] : 1.f, y[((size_t)t * top + j) * width + i], v);
+    for (int j = 0; j < top; ++j) {
+      // a choice past the experts is an identity expert: its output is the token's input
+      const bool same = ids != nullptr && ids[(size_t)t * top + j] >= n_experts;
+      const float yj = same ? to_f32(x_in[(size_t)t * ldx + i]) : y[((size_t)t * top + j) * width + i];
+      v = fmaf(weights ? weights[(size_t)t * top + j] : 1.f, yj, v);
+    }
     if (shared) v = fmaf(sg, to_f32(shared[(size_t)t * width + i]), v);
     out[(size_t)t * width + i] = from_f32<T>(v);
   }
@@ -374,7 +514,8 @@ __global__ void __launch_bounds__(256)
 template <typename T, int KEEP>
 __global__ void __launch_bounds__(256)
     combine_small_kernel(const float* __restrict__ y, const float* __restrict__ weights, int top, const T* __restrict__ shared,
-                         const float* __restrict__ shared_gate, long ldg, T* __restrict__ out, int width) {
+                         const float* __restrict__ shared_gate, long ldg, T* __restrict__ out, int width, const int* __restrict__ ids,
+                         int n_experts, const T* __restrict__ x_in, long ldx) {
   const int t = blockIdx.x;
   f32x4 acc[KEEP], sh[KEEP];
 #pragma unroll
@@ -395,11 +536,19 @@ __global__ void __launch_bounds__(256)
   for (int j = 0; j < top; ++j) {
     const float wj = weights ? weights[(size_t)t * top + j] : 1.f;  // no weights: the plain sum
     const float* row = y + ((size_t)t * top + j) * width;
+    // a choice past the experts is an identity expert: its output is the token's input
+    const bool same = ids != nullptr && ids[(size_t)t * top + j] >= n_experts;
 #pragma unroll
     for (int n = 0; n < KEEP; ++n) {
       const int i = (threadIdx.x + n * 256) * 4;
       if (i < width) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(row + i);
+        f32x4 v;
+        if (same) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = to_f32(x_in[(size_t)t * ldx + i + e]);
+        } else {
+          v = *reinterpret_cast<const f32x4*>(row + i);
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[n][e] = fmaf(wj, v[e], acc[n][e]);
       }
@@ -422,17 +571,19 @@ __global__ void __launch_bounds__(256)
 }
 
 extern "C" int fmsamd_moe_combine(const float* y, const float* weights, int top, const void* shared, const float* shared_gate,
-                                  long ldg, void* out, int dtype, int n_tokens, int width, hipStream_t stream) {
+                                  long ldg, void* out, int dtype, int n_tokens, int width, const int* ids, int n_experts,
+                                  const void* x_in, long ldx, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && top > 0 && width > 0, "moe_combine: bad sizes T=%d top=%d width=%d", n_tokens, top, width);
+  FMS_REQUIRE(ids == nullptr || (x_in != nullptr && ldx >= width && n_experts >= 0), "moe_combine: identity experts need the tokens' inputs");
   if (width <= 1024 * 4 && width % 4 == 0 && dtype == FMS_F32)
-    combine_small_kernel<float, 4><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const float*)shared, shared_gate, ldg, (float*)out, width);
+    combine_small_kernel<float, 4><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const float*)shared, shared_gate, ldg, (float*)out, width, ids, n_experts, (const float*)x_in, ldx);
   else if (width <= 1024 * 4 && width % 4 == 0 && dtype == FMS_BF16)
-    combine_small_kernel<bf16, 4><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const bf16*)shared, shared_gate, ldg, (bf16*)out, width);
+    combine_small_kernel<bf16, 4><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const bf16*)shared, shared_gate, ldg, (bf16*)out, width, ids, n_experts, (const bf16*)x_in, ldx);
   else if (dtype == FMS_F32)
-    combine_kernel<float><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const float*)shared, shared_gate, ldg, (float*)out, width);
+    combine_kernel<float><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const float*)shared, shared_gate, ldg, (float*)out, width, ids, n_experts, (const float*)x_in, ldx);
   else if (dtype == FMS_BF16)
-    combine_kernel<bf16><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const bf16*)shared, shared_gate, ldg, (bf16*)out, width);
+    combine_kernel<bf16><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const bf16*)shared, shared_gate, ldg, (bf16*)out, width, ids, n_experts, (const bf16*)x_in, ldx);
   else
     FMS_REQUIRE(false, "moe_combine: unknown dtype %d", dtype);
   FMS_LAUNCH_CHECK("moe_combine");

@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define FMSAMD_ABI_VERSION 4
+#define FMSAMD_ABI_VERSION 5
 
 // element types
 #define FMS_F32 0
@@ -178,6 +178,9 @@ int fmsamd_norm_add_norm(float* resid, const void* branch, int act_dtype, const 
 // out[t, 0:n] = x[t, col0 : col0 + n] / rms * weight for float32 rows ldx apart
 int fmsamd_rms_norm_cols(const float* x, long ldx, int col0, int n, const void* weight, int weight_dtype, float eps,
                          void* out, int out_dtype, long ldo, int rows, hipStream_t stream);
+// out[t, 0:n] = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e (powers element by element) for float32 rows ldz apart
+int fmsamd_poly_norm(const float* z, long ldz, int n, float a, float b, float c, float e, float eps, void* out, int out_dtype,
+                     long ldo, int rows, hipStream_t stream);
 // out = act(x), act one of FMS_ACT_*
 int fmsamd_activate(const void* x, void* out, int dtype, long n, int act, hipStream_t stream);
 // gu [T, 2 * hidden] (gate first): out = g' sigmoid(alpha g') (u' + shift), g' = min(g, limit), u' = clamp(u, +-limit)
@@ -235,12 +238,20 @@ int fmsamd_moe_group(const int* ids, int n_pairs, int n_experts, int* order, int
                      hipStream_t stream);
 // stage 0: y[sorted pair] = act(s x Wg^T, s x Wu^T) (w1, w2 = gate, up [E, N, K]; s = in_scale[pair], or 1 if null: a
 // weight on the expert's input, applied to the float32 sums); stage 1: y[pair] = x W^T, float32
+// With w2 null at stage 0 the experts have no gate: y[sorted pair] = act(s x W1^T), act one of FMS_ACT_*.
 int fmsamd_moe_experts(int stage, const void* x, long ldx, const void* w1, const void* w2, void* y, int dtype,
                        const int* order, const int* tiles, int max_tiles, int tile_rows, int top, int N, int K, float limit,
-                       float alpha, float shift, const float* in_scale, hipStream_t stream);
-// weights null: the plain sum of a token's rows
+                       float alpha, float shift, const float* in_scale, int act, hipStream_t stream);
+// weights null: the plain sum of a token's rows.  ids (or null) [T, top] with n_experts: a choice of n_experts or more is
+// an identity expert, whose output is the token's input x_in [T, ldx] (of the output's type) instead of a row of y.
 int fmsamd_moe_combine(const float* y, const float* weights, int top, const void* shared, const float* shared_gate, long ldg,
-                       void* out, int dtype, int n_tokens, int width, hipStream_t stream);
+                       void* out, int dtype, int n_tokens, int width, const int* ids, int n_experts, const void* x_in, long ldx,
+                       hipStream_t stream);
+// Routing over groups: s = softmax over all n_outputs logits; outputs are chosen by s + correction (float32 [n_outputs] or
+// null) among the `keep` groups (of `groups` equal runs of neighbours) whose largest choice score is largest; the weights
+// are the chosen outputs' s over their sum (+ 1e-20), times scale.
+int fmsamd_moe_route_grouped(const float* logits, long ld, int n_tokens, int n_outputs, int top, const float* correction,
+                             int groups, int keep, float scale, int* ids, float* weights, hipStream_t stream);
 
 // ---- steps around attention (attention_extras.hip) ------------------------------------------------------------------
 // float32 rows [q (nq) | k (nk) | v (nv)]: out = [q / rms(q) * wq | k / rms(k) * wk | v], each norm over its whole run of
@@ -276,6 +287,35 @@ int fmsamd_delta_rule(const float* qkv, const float* beta, const float* decay, c
 int fmsamd_gated_head_norm(const float* o, const float* gate, long ldg, const void* weight, int weight_dtype, float eps,
                            int act, float out_scale, void* out, int out_dtype, long ldo, const int* seq_of_token,
                            int n_tokens, int heads, int vdim, hipStream_t stream);
+
+// ---- norms behind the branches only, short convolutions (post_norm.hip) --------------------------------------------
+// resid += gnorm(branch) * branch_weight (branch null: nothing is added; written back unless `rows` is given), where gnorm
+// divides each of branch_groups equal consecutive parts of a row by its own root mean square (branch_groups 0: the branch
+// is added as it is); then out is nothing, the
+// stream in the activation type, or gnorm(resid) * weight with `groups` parts.
+#define FMS_CHAIN_NONE 0
+#define FMS_CHAIN_CAST 1
+#define FMS_CHAIN_NORM 2
+int fmsamd_group_norm_chain(float* resid, const void* branch, int act_dtype, const void* branch_weight, int branch_weight_dtype,
+                            int branch_groups, float branch_eps, const void* weight, int weight_dtype, int groups, float eps,
+                            void* out, int out_mode, const int* rows, int n_out, int width, hipStream_t stream);
+// out[t, c] = (x[t, c] if add_input) + bias[c] + sum_j conv_w[c, j] x[t - taps + 1 + j, c] over a sequence's own tokens; the
+// inputs before the step come from conv_state [slots][taps-1][channels] (float32), which is then moved on.  x: float32 rows.
+int fmsamd_short_conv(const float* x, long ld, int channels, const void* conv_w, const void* bias, int weight_dtype, int taps,
+                      float* conv_state, const int* seq_of_token, const int* slot_ids, int add_input, void* out, int out_dtype,
+                      long ldo, int n_tokens, hipStream_t stream);
+
+// ---- the real-gated linear recurrent unit (rglru.hip) -------------------------------------------------------------------
+// u: float32 rows; ra_t, ri_t [blocks][in][out] (transposed square matrices), ra_b, ri_b, lam float32 [channels];
+// a = exp(-c sigmoid(Ra u + ba) softplus(lam)), b = sqrt(1 - a^2) sigmoid(Ri u + bi) u, both float32 [T, channels].
+int fmsamd_rglru_gates(const float* u, long ldu, const void* ra_t, const float* ra_b, const void* ri_t, const float* ri_b,
+                       int weight_dtype, const float* lam, float c, const int* seq_of_token, float* a_out, float* b_out,
+                       int n_tokens, int channels, int blocks, hipStream_t stream);
+// S <- a S + b over every sequence's tokens of the step (seq_starts [n_seqs + 1]), from and into state [slots][channels];
+// out[t] = S * act(y[t]) (y: float32 rows ldy apart).
+int fmsamd_rglru_scan(const float* a, const float* b, const float* y, long ldy, int act, float* state, const int* seq_starts,
+                      const int* seq_of_token, const int* slot_ids, void* out, int out_dtype, long ldo, int n_seqs, int channels,
+                      hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -4,6 +4,7 @@
 //       stream += branch / rms(branch) * wb;   out = stream / rms(stream) * w
 //     in one pass over the row: two row norms and the residual sum, all float32.
 //   rms_norm_cols: the RMS norm of a run of columns of float32 rows (a slice of a fused projection).
+//   poly_norm: a sum of the RMS-normed first three powers of a token's values.
 //   activate: out = act(x), the activations of common.h.
 //   clamped_gated_act: out = g' * sigmoid(alpha g') * (u' + shift), g' = min(g, limit), u' = clamp(u, -limit, limit).
 #include "common.h"
@@ -178,6 +179,45 @@ extern "C" int fmsamd_rms_norm_cols(const float* x, long ldx, int col0, int n, c
   else
     FMS_REQUIRE(false, "rms_norm_cols: unknown dtype %d", out_dtype);
   FMS_LAUNCH_CHECK("rms_norm_cols");
+  return 0;
+}
+
+// out[t, :] = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e over a token's n values (powers element by element,
+// eps inside every root): z float32 rows ldz apart.  One block per row; the three sums of squares are float32.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    poly_norm_kernel(const float* __restrict__ z, long ldz, int n, float a, float b, float c, float e, float eps,
+                     T* __restrict__ out, long ldo) {
+  __shared__ float scratch[17];
+  const float* zr = z + (size_t)blockIdx.x * ldz;
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = zr[i], v2 = v * v, v3 = v2 * v;
+    s2 = fmaf(v, v, s2);
+    s4 = fmaf(v2, v2, s4);
+    s6 = fmaf(v3, v3, s6);
+  }
+  const float r1 = a * rsqrtf(block_sum(s2, scratch) / (float)n + eps);
+  const float r2 = b * rsqrtf(block_sum(s4, scratch) / (float)n + eps);
+  const float r3 = c * rsqrtf(block_sum(s6, scratch) / (float)n + eps);
+  T* o = out + (size_t)blockIdx.x * ldo;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = zr[i], v2 = v * v;
+    o[i] = from_f32<T>(fmaf(r1, v, fmaf(r2, v2, fmaf(r3, v2 * v, e))));
+  }
+}
+
+extern "C" int fmsamd_poly_norm(const float* z, long ldz, int n, float a, float b, float c, float e, float eps, void* out,
+                                int out_dtype, long ldo, int rows, hipStream_t stream) {
+  if (rows == 0) return 0;
+  FMS_REQUIRE(rows > 0 && n > 0 && ldz >= n && ldo >= n, "poly_norm: bad sizes rows=%d n=%d ldz=%ld ldo=%ld", rows, n, ldz, ldo);
+  if (out_dtype == FMS_F32)
+    poly_norm_kernel<float><<<rows, 256, 0, stream>>>(z, ldz, n, a, b, c, e, eps, (float*)out, ldo);
+  else if (out_dtype == FMS_BF16)
+    poly_norm_kernel<bf16><<<rows, 256, 0, stream>>>(z, ldz, n, a, b, c, e, eps, (bf16*)out, ldo);
+  else
+    FMS_REQUIRE(false, "poly_norm: unknown dtype %d", out_dtype);
+  FMS_LAUNCH_CHECK("poly_norm");
   return 0;
 }
 

@@ -1,0 +1,158 @@
+// What a block needs whose norms sit behind its branches only, and whose branches read the stream itself.
+//
+//   group_norm_chain: stream += gnorm_b(branch) * wb (or the branch as it is);   out = nothing | the stream as it is | gnorm(stream) * w
+//     gnorm splits a row into `groups` equal consecutive parts and divides each by its own root mean square
+//     (eps inside the root); one group is the plain RMS norm.  Both statistics and the sum are float32.
+//   short_conv: out = (x +) conv(x) (+ bias): a causal convolution over time on every channel, the inputs before the
+//     step taken from the sequence's state; then the state is moved on (short_conv.h).
+#include "common.h"
+#include "fmsamd.h"
+#include "short_conv.h"
+
+__device__ __forceinline__ float scale_at(const void* w, int dtype, int i) {
+  if (w == nullptr) return 1.f;
+  return dtype == FMS_F32 ? ((const float*)w)[i] : (float)((const bf16*)w)[i];
+}
+
+// inv[g] = rsqrt(mean(row[g's part]^2) + eps): a wave a group, the lanes strided over the part, so that the order of the
+// sum depends on nothing but the sizes.
+__device__ __forceinline__ void group_scales(const float* row, float* inv, int width, int groups, float eps) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  const int part = width / groups;
+  for (int g = wave; g < groups; g += nwaves) {
+    const float* p = row + (size_t)g * part;
+    float sq = 0.f;
+    for (int i = lane; i < part; i += WAVE) sq = fmaf(p[i], p[i], sq);
+    sq = wave_sum(sq);
+    if (lane == 0) inv[g] = rsqrtf(sq / (float)part + eps);
+  }
+}
+
+// One block per output row; the row waits in LDS (width floats, then the groups' scales).
+template <typename T>
+__global__ void __launch_bounds__(256)
+    group_norm_chain_kernel(float* __restrict__ resid, const T* __restrict__ branch, const void* __restrict__ wb, int wb_dtype,
+                            int groups_b, float eps_b, const void* __restrict__ w, int w_dtype, int groups, float eps,
+                            T* __restrict__ out, int out_mode, const int* __restrict__ rows, int width) {
+  extern __shared__ float lds[];
+  float* row = lds;
+  float* inv = lds + width;
+  const int r = rows ? rows[blockIdx.x] : blockIdx.x;
+  float* x = resid + (size_t)r * width;
+  if (branch != nullptr) {
+    const T* b = branch + (size_t)r * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) row[i] = to_f32(b[i]);
+    if (groups_b > 0) {
+      __syncthreads();
+      group_scales(row, inv, width, groups_b, eps_b);
+      __syncthreads();
+    }
+    const int part = groups_b > 0 ? width / groups_b : width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+      const float v = x[i] + (groups_b > 0 ? row[i] * inv[i / part] * scale_at(wb, wb_dtype, i) : row[i]);
+      row[i] = v;
+      if (!rows) x[i] = v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < width; i += blockDim.x) row[i] = x[i];
+  }
+  if (out_mode == FMS_CHAIN_NONE) return;
+  T* o = out + (size_t)blockIdx.x * width;
+  if (out_mode == FMS_CHAIN_CAST) {
+    for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = from_f32<T>(row[i]);  // a thread reads what it wrote
+    return;
+  }
+  __syncthreads();
+  group_scales(row, inv, width, groups, eps);
+  __syncthreads();
+  const int part = width / groups;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = from_f32<T>(row[i] * inv[i / part] * scale_at(w, w_dtype, i));
+}
+
+extern "C" int fmsamd_group_norm_chain(float* resid, const void* branch, int act_dtype, const void* branch_weight,
+                                       int branch_weight_dtype, int branch_groups, float branch_eps, const void* weight,
+                                       int weight_dtype, int groups, float eps, void* out, int out_mode, const int* rows,
+                                       int n_out, int width, hipStream_t stream) {
+  if (n_out == 0) return 0;
+  FMS_REQUIRE(n_out > 0 && width > 0 && width <= 15360, "group_norm_chain: bad sizes rows=%d width=%d", n_out, width);
+  FMS_REQUIRE(resid != nullptr, "group_norm_chain: the stream is needed");
+  FMS_REQUIRE(out_mode >= FMS_CHAIN_NONE && out_mode <= FMS_CHAIN_NORM && (out_mode == FMS_CHAIN_NONE || out != nullptr),
+              "group_norm_chain: output mode %d", out_mode);
+  FMS_REQUIRE(branch == nullptr || branch_groups == 0 || (branch_groups > 0 && branch_groups <= 1024 && width % branch_groups == 0),
+              "group_norm_chain: %d groups do not divide the branch's %d channels", branch_groups, width);
+  FMS_REQUIRE(out_mode != FMS_CHAIN_NORM || (groups > 0 && groups <= 1024 && width % groups == 0),
+              "group_norm_chain: %d groups do not divide %d channels", groups, width);
+  const size_t lds = ((size_t)width + 1024) * sizeof(float);
+  if (act_dtype == FMS_F32)
+    group_norm_chain_kernel<float><<<n_out, 256, lds, stream>>>(resid, (const float*)branch, branch_weight, branch_weight_dtype,
+                                                                branch_groups, branch_eps, weight, weight_dtype, groups, eps,
+                                                                (float*)out, out_mode, rows, width);
+  else if (act_dtype == FMS_BF16)
+    group_norm_chain_kernel<bf16><<<n_out, 256, lds, stream>>>(resid, (const bf16*)branch, branch_weight, branch_weight_dtype,
+                                                               branch_groups, branch_eps, weight, weight_dtype, groups, eps,
+                                                               (bf16*)out, out_mode, rows, width);
+  else
+    FMS_REQUIRE(false, "group_norm_chain: unknown dtype %d", act_dtype);
+  FMS_LAUNCH_CHECK("group_norm_chain");
+  return 0;
+}
+
+// A block per token, a thread per channel and pass; all taps of a channel are asked for before any is used.
+template <typename W, typename T>
+__global__ void __launch_bounds__(1024)
+    short_conv_kernel(const float* __restrict__ x, long ld, int C, const W* __restrict__ conv_w, const W* __restrict__ bias,
+                      int taps, const float* __restrict__ conv_state, const int* __restrict__ seq_of_token,
+                      const int* __restrict__ slot_ids, int add_input, T* __restrict__ out, long ldo) {
+  const int t = blockIdx.x;
+  const int seq = seq_of_token[t];
+  T* o = out + (size_t)t * ldo;
+  if (seq < 0) {  // a padding row: zeros, so that whatever reads the row reads numbers
+    for (int c = threadIdx.x; c < C; c += blockDim.x) o[c] = from_f32<T>(0.f);
+    return;
+  }
+  const int have = tokens_before(seq_of_token, t, seq, taps);
+  const float* state = conv_state + (size_t)slot_ids[seq] * (taps - 1) * C;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float xs[CONV_MAX_TAPS], ws[CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+      const int d = taps - 1 - j;  // how far back this tap reaches
+      xs[j] = ws[j] = 0.f;
+      if (j < taps) {
+        xs[j] = d <= have ? x[(size_t)(t - d) * ld + c] : state[(size_t)(taps - 1 + have - d) * C + c];
+        ws[j] = to_f32(conv_w[(size_t)c * taps + j]);
+      }
+    }
+    float acc = bias ? to_f32(bias[c]) : 0.f;
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) acc = fmaf(ws[j], xs[j], acc);
+    if (add_input) acc += x[(size_t)t * ld + c];
+    o[c] = from_f32<T>(acc);
+  }
+}
+
+extern "C" int fmsamd_short_conv(const float* x, long ld, int channels, const void* conv_w, const void* bias, int weight_dtype,
+                                 int taps, float* conv_state, const int* seq_of_token, const int* slot_ids, int add_input,
+                                 void* out, int out_dtype, long ldo, int n_tokens, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && channels > 0 && ld >= channels && ldo >= channels, "short_conv: bad sizes T=%d C=%d ld=%ld ldo=%ld",
+              n_tokens, channels, ld, ldo);
+  FMS_REQUIRE(taps >= 1 && taps <= CONV_MAX_TAPS, "short_conv: %d taps (1 to %d)", taps, CONV_MAX_TAPS);
+  FMS_REQUIRE(taps == 1 || conv_state != nullptr, "short_conv: a convolution of %d taps needs the sequences' state", taps);
+  const int threads = n_tokens <= 64 ? 1024 : 256;
+#define FMS_CONV(W, T)                                                                                                     \
+  short_conv_kernel<W, T><<<n_tokens, threads, 0, stream>>>(x, ld, channels, (const W*)conv_w, (const W*)bias, taps, conv_state, \
+                                                            seq_of_token, slot_ids, add_input, (T*)out, ldo)
+  if (weight_dtype == FMS_F32 && out_dtype == FMS_F32) FMS_CONV(float, float);
+  else if (weight_dtype == FMS_F32 && out_dtype == FMS_BF16) FMS_CONV(float, bf16);
+  else if (weight_dtype == FMS_BF16 && out_dtype == FMS_F32) FMS_CONV(bf16, float);
+  else if (weight_dtype == FMS_BF16 && out_dtype == FMS_BF16) FMS_CONV(bf16, bf16);
+  else FMS_REQUIRE(false, "short_conv: unknown dtypes %d %d", weight_dtype, out_dtype);
+#undef FMS_CONV
+  FMS_LAUNCH_CHECK("short_conv");
+  if (taps > 1) {
+    conv_state_kernel<<<n_tokens, threads, 0, stream>>>(x, ld, taps, conv_state, seq_of_token, slot_ids, n_tokens, channels);
+    FMS_LAUNCH_CHECK("conv_state");
+  }
+  return 0;
+}

@@ -58,6 +58,11 @@ class DecoderModel(Part):
                 if need is None or other != need:
                     raise ValueError(f"schedule entry {n} cannot read the cache of entry {entry.cache_of}: their needs differ")
             sneed = mixer.state_need()
+            # a block may keep state of its own beside its mixer's (the last rows of the stream that a convolution on the
+            # mixer's input reads); every run of a layer has its own
+            block_need = getattr(self.layers[entry.layer], "state_need", lambda: None)()
+            if block_need is not None:
+                sneed = StateNeed(tuple(block_need.tensors) + (tuple(sneed.tensors) if sneed is not None else ()))
             if sneed is not None:
                 state.append((n, sneed))
         return kv, state

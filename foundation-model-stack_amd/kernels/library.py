@@ -17,7 +17,7 @@ import torch  # noqa: F401  (loads libamdhip64 before our library asks for it)
 
 from . import build as _build
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
@@ -58,7 +58,13 @@ _SIGNATURES = {
     "fmsamd_latent_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P],
     "fmsamd_moe_route": [P, L, I, I, I, I, P, P, P],
     "fmsamd_moe_group": [P, I, I, P, P, I, I, P],
-    "fmsamd_moe_experts": [I, P, L, P, P, P, I, P, P, I, I, I, I, I, F, F, F, P, P],
+    "fmsamd_moe_experts": [I, P, L, P, P, P, I, P, P, I, I, I, I, I, F, F, F, P, I, P],
+    "fmsamd_moe_route_grouped": [P, L, I, I, I, P, I, I, F, P, P, P],
+    "fmsamd_poly_norm": [P, L, I, F, F, F, F, F, P, I, L, I, P],
+    "fmsamd_group_norm_chain": [P, P, I, P, I, I, F, P, I, I, F, P, I, P, I, I, P],
+    "fmsamd_short_conv": [P, L, I, P, P, I, I, P, P, P, I, P, I, L, I, P],
+    "fmsamd_rglru_gates": [P, L, P, P, P, P, I, P, F, P, P, P, I, I, I, P],
+    "fmsamd_rglru_scan": [P, P, P, L, I, P, P, P, P, P, I, L, I, I, P],
     "fmsamd_qk_projection_norm": [P, L, I, I, I, P, P, I, F, P, I, L, P, I, P],
     "fmsamd_gate_mul": [P, L, P, L, I, F, P, L, I, I, I, P],
     "fmsamd_scale_f32": [P, L, F, P],
@@ -66,7 +72,7 @@ _SIGNATURES = {
     "fmsamd_delta_prepare": [P, L, I, P, L, I, P, I, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, P],
     "fmsamd_delta_rule": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
     "fmsamd_gated_head_norm": [P, P, L, P, I, F, I, F, P, I, L, P, I, I, I, P],
-    "fmsamd_moe_combine": [P, P, I, P, P, L, P, I, I, I, P],
+    "fmsamd_moe_combine": [P, P, I, P, P, L, P, I, I, I, P, I, P, L, P],
     "fmsamd_probe_read": [P, L, I, I, P, P],
     "fmsamd_probe_mfma": [I, I, I, P, P, P],
 }

@@ -661,6 +661,140 @@ def rms_norm_cols(x: torch.Tensor, col0: int, n: int, weight: Optional[torch.Ten
     return out
 
 
+def poly_norm(z: torch.Tensor, coefficients, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """a N(z) + b N(z^2) + c N(z^3) + e for coefficients (a, b, c, e), powers element by element, N a row divided by its
+    root mean square: float32 rows [T, n] -> [T, n] in out_dtype."""
+    _need_cuda(z)
+    _rows2d("z", z)
+    if z.dtype != torch.float32:
+        raise ValueError("poly_norm takes float32 rows")
+    a, b, c, e = (float(v) for v in coefficients)
+    out = torch.empty(z.shape[0], z.shape[1], dtype=out_dtype, device=z.device)
+    check(load().fmsamd_poly_norm(z.data_ptr(), z.stride(0), z.shape[1], a, b, c, e, float(eps), out.data_ptr(), _code(out_dtype),
+                                  out.stride(0), z.shape[0], _stream()))
+    return out
+
+
+CHAIN_NONE, CHAIN_CAST, CHAIN_NORM = 0, 1, 2
+
+
+def group_norm_chain(resid: torch.Tensor, branch: Optional[torch.Tensor], branch_weight: Optional[torch.Tensor], branch_groups: int,
+                     branch_eps: float, act_dtype: torch.dtype, out_mode: int = CHAIN_NONE, weight: Optional[torch.Tensor] = None,
+                     groups: int = 1, eps: float = 0.0, rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """resid += gnorm(branch) * branch_weight (float32, in place unless `rows` is given; branch None: nothing is added), gnorm
+    dividing each of `branch_groups` equal consecutive parts of a row by its own root mean square (0: the branch is added
+    as it is).  Returns nothing
+    (CHAIN_NONE), the stream in act_dtype (CHAIN_CAST), or gnorm(resid) * weight with `groups` parts (CHAIN_NORM); only
+    `rows` if given."""
+    _need_cuda(resid, branch, branch_weight, weight, rows)
+    if resid.dtype != torch.float32 or resid.dim() != 2 or not resid.is_contiguous():
+        raise ValueError("the residual stream must be a contiguous float32 [T, width] tensor")
+    T, width = resid.shape
+    if branch is not None and (branch.shape != resid.shape or not branch.is_contiguous() or branch.dtype != act_dtype):
+        raise ValueError(f"branch must be contiguous {tuple(resid.shape)} of {act_dtype}, got {tuple(branch.shape)} {branch.dtype}")
+    for name, t in (("branch weight", branch_weight), ("weight", weight)):
+        if t is not None and (t.shape != (width,) or not t.is_contiguous()):
+            raise ValueError(f"norm {name} must be a contiguous [{width}] tensor, got {tuple(t.shape)}")
+    if branch is not None and branch_groups != 0 and (branch_groups < 1 or width % branch_groups):
+        raise ValueError(f"{branch_groups} groups do not divide {width} channels")
+    if out_mode == CHAIN_NORM and (groups < 1 or width % groups):
+        raise ValueError(f"{groups} groups do not divide {width} channels")
+    n_out = T
+    if rows is not None:
+        _need_i32("rows", rows)
+        n_out = rows.numel()
+    out = torch.empty(n_out, width, dtype=act_dtype, device=resid.device) if out_mode != CHAIN_NONE else None
+    check(load().fmsamd_group_norm_chain(resid.data_ptr(), _ptr(branch), _code(act_dtype), _ptr(branch_weight),
+                                         _code(branch_weight.dtype) if branch_weight is not None else 0, int(branch_groups), float(branch_eps),
+                                         _ptr(weight), _code(weight.dtype) if weight is not None else 0, int(groups), float(eps),
+                                         _ptr(out), int(out_mode), _ptr(rows), n_out, width, _stream()))
+    return out
+
+
+CONV_MAX_TAPS = 8
+
+
+def short_conv(x: torch.Tensor, col0: int, channels: int, conv_w: torch.Tensor, bias: Optional[torch.Tensor], conv_state: Optional[torch.Tensor],
+               seq_of_token: torch.Tensor, slot_ids: torch.Tensor, out_dtype: torch.dtype, add_input: bool = False) -> torch.Tensor:
+    """A causal convolution over time on the channels col0 .. col0 + channels of float32 rows: out[t, c] = (x[t, c] if
+    add_input) + bias[c] + sum_j conv_w[c, j] x[t - taps + 1 + j, c] over the sequence's own tokens -> [T, channels] in
+    out_dtype.  The inputs before the step come from conv_state [slots, taps - 1, channels] (float32; zeros before a
+    sequence's start), which is then moved on to the step's last inputs."""
+    _need_cuda(x, conv_w, bias, conv_state, seq_of_token, slot_ids)
+    _rows2d("x", x)
+    _need_i32("seq_of_token", seq_of_token)
+    _need_i32("slot_ids", slot_ids)
+    T = x.shape[0]
+    if x.dtype != torch.float32 or col0 < 0 or channels <= 0 or col0 + channels > x.shape[1] or seq_of_token.numel() < T:
+        raise ValueError("short_conv takes float32 rows that hold the channels asked for, and a sequence index per token")
+    if conv_w.dim() != 2 or conv_w.shape[0] != channels or not conv_w.is_contiguous() or not 1 <= conv_w.shape[1] <= CONV_MAX_TAPS:
+        raise ValueError(f"the convolution's weights are contiguous [{channels}, taps], taps at most {CONV_MAX_TAPS}")
+    taps = conv_w.shape[1]
+    if bias is not None and (tuple(bias.shape) != (channels,) or not bias.is_contiguous() or bias.dtype != conv_w.dtype):
+        raise ValueError(f"the convolution's bias is a contiguous [{channels}] tensor of the weights' type")
+    if taps > 1 and (conv_state is None or conv_state.dtype != torch.float32 or conv_state.dim() != 3
+                     or tuple(conv_state.shape[1:]) != (taps - 1, channels) or not conv_state.is_contiguous()):
+        raise ValueError(f"the convolution's state is contiguous float32 [slots, {taps - 1}, {channels}]")
+    out = torch.empty(T, channels, dtype=out_dtype, device=x.device)
+    view = x[:, col0 : col0 + channels]
+    check(load().fmsamd_short_conv(view.data_ptr(), x.stride(0), channels, conv_w.data_ptr(), _ptr(bias), _code(conv_w.dtype), taps,
+                                   _ptr(conv_state), seq_of_token.data_ptr(), slot_ids.data_ptr(), int(bool(add_input)), out.data_ptr(),
+                                   _code(out_dtype), out.stride(0), T, _stream()))
+    return out
+
+
+def rglru_gates(u: torch.Tensor, ra_t: torch.Tensor, ra_b: torch.Tensor, ri_t: torch.Tensor, ri_b: torch.Tensor, lam: torch.Tensor,
+                c: float, seq_of_token: torch.Tensor):
+    """The gates of the real-gated linear recurrent unit, from float32 rows u [T, channels]: with block-diagonal Ra, Ri given
+    as [blocks, in, out] (each block transposed), a = exp(-c sigmoid(Ra u + ra_b) softplus(lam)) and
+    b = sqrt(1 - a^2) sigmoid(Ri u + ri_b) u, both float32 [T, channels]."""
+    _need_cuda(u, ra_t, ra_b, ri_t, ri_b, lam, seq_of_token)
+    _rows2d("u", u)
+    _need_i32("seq_of_token", seq_of_token)
+    T, C = u.shape
+    if u.dtype != torch.float32 or seq_of_token.numel() < T:
+        raise ValueError("rglru_gates takes float32 rows and a sequence index per token")
+    if ra_t.dim() != 3 or ra_t.shape[1] != ra_t.shape[2] or ra_t.shape[0] * ra_t.shape[1] != C or ra_t.shape != ri_t.shape \
+            or ra_t.dtype != ri_t.dtype or not (ra_t.is_contiguous() and ri_t.is_contiguous()):
+        raise ValueError(f"the gates' matrices are contiguous [blocks, n, n] with blocks * n = {C}, of one type")
+    for name, t in (("ra_b", ra_b), ("ri_b", ri_b), ("lam", lam)):
+        if t.dtype != torch.float32 or tuple(t.shape) != (C,) or not t.is_contiguous():
+            raise ValueError(f"{name} is a contiguous float32 [{C}] tensor")
+    a = torch.empty(T, C, dtype=torch.float32, device=u.device)
+    b = torch.empty(T, C, dtype=torch.float32, device=u.device)
+    check(load().fmsamd_rglru_gates(u.data_ptr(), u.stride(0), ra_t.data_ptr(), ra_b.data_ptr(), ri_t.data_ptr(), ri_b.data_ptr(),
+                                    _code(ra_t.dtype), lam.data_ptr(), float(c), seq_of_token.data_ptr(), a.data_ptr(), b.data_ptr(), T, C,
+                                    ra_t.shape[0], _stream()))
+    return a, b
+
+
+def rglru_scan(a: torch.Tensor, b: torch.Tensor, y: torch.Tensor, activation: str, state: torch.Tensor, seq_starts: torch.Tensor,
+               seq_of_token: torch.Tensor, slot_ids: torch.Tensor, n_seqs: int, out_dtype: torch.dtype, zero_rows: bool = False) -> torch.Tensor:
+    """S <- a S + b over the tokens of every sequence of the step, from and into state [slots, channels] (float32);
+    out[t] = S * activation(y[t]) in out_dtype.  a, b: contiguous float32 [T, channels]; y: float32 rows [T, channels] of
+    any stride.  Sequence s owns the token rows seq_starts[s] .. seq_starts[s + 1] and the state of slot_ids[s].
+    zero_rows: rows that belong to no sequence come back as zeros."""
+    _need_cuda(a, b, y, state, seq_starts, seq_of_token, slot_ids)
+    _rows2d("y", y)
+    for name, t in (("seq_starts", seq_starts), ("seq_of_token", seq_of_token), ("slot_ids", slot_ids)):
+        _need_i32(name, t)
+    T, C = a.shape
+    for name, t in (("a", a), ("b", b)):
+        if t.dtype != torch.float32 or tuple(t.shape) != (T, C) or not t.is_contiguous():
+            raise ValueError(f"{name} is contiguous float32 [{T}, {C}]")
+    if y.dtype != torch.float32 or tuple(y.shape) != (T, C):
+        raise ValueError(f"y is float32 [{T}, {C}]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != C or not state.is_contiguous():
+        raise ValueError(f"the state is contiguous float32 [slots, {C}]")
+    if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs or seq_of_token.numel() < T:
+        raise ValueError("the step's index arrays are shorter than its sequences or tokens")
+    out = (torch.zeros if zero_rows else torch.empty)(T, C, dtype=out_dtype, device=a.device)
+    check(load().fmsamd_rglru_scan(a.data_ptr(), b.data_ptr(), y.data_ptr(), y.stride(0), ACTIVATIONS[activation], state.data_ptr(),
+                                   seq_starts.data_ptr(), seq_of_token.data_ptr(), slot_ids.data_ptr(), out.data_ptr(), _code(out_dtype),
+                                   out.stride(0), int(n_seqs), C, _stream()))
+    return out
+
+
 def activation(x: torch.Tensor, kind: str) -> torch.Tensor:
     """act(x), elementwise, for the activations of ACTIVATIONS."""
     _need_cuda(x)
@@ -847,12 +981,40 @@ def moe_route(logits: torch.Tensor, n_experts: int, top: int, score: str = "soft
     return ids, weights
 
 
-def moe_experts(x: torch.Tensor, ids: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor,
-                limit: float, alpha: float, shift: float, in_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+def moe_route_grouped(logits: torch.Tensor, n_outputs: int, top: int, correction: Optional[torch.Tensor] = None, groups: int = 1,
+                      keep: int = 1, scale: float = 1.0):
+    """float32 logits [T, >= n_outputs] -> (int32 ids [T, top], float32 weights [T, top]).  s = softmax over the first
+    n_outputs columns; an output is chosen by s + correction (float32 [n_outputs]) but weighted by s; the outputs form
+    `groups` equal runs of neighbours, a group's score is its largest choice score, and only outputs of the `keep` best
+    groups can be chosen; the weights are the chosen s over their sum (+ 1e-20), times `scale`."""
+    _need_cuda(logits, correction)
+    _rows2d("logits", logits)
+    if logits.dtype != torch.float32 or logits.shape[1] < n_outputs:
+        raise ValueError("router logits are float32 [T, >= outputs]")
+    if correction is not None and (correction.dtype != torch.float32 or tuple(correction.shape) != (n_outputs,) or not correction.is_contiguous()):
+        raise ValueError(f"the correction is a contiguous float32 [{n_outputs}] tensor")
+    if groups < 1 or n_outputs % groups or not 1 <= keep <= groups or keep * (n_outputs // groups) < top:
+        raise ValueError(f"{groups} groups over {n_outputs} outputs with {keep} kept cannot give {top} choices")
+    T = logits.shape[0]
+    ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    weights = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    check(load().fmsamd_moe_route_grouped(logits.data_ptr(), logits.stride(0), T, n_outputs, top, _ptr(correction), groups, keep,
+                                          float(scale), ids.data_ptr(), weights.data_ptr(), _stream()))
+    return ids, weights
+
+
+def moe_experts(x: torch.Tensor, ids: torch.Tensor, gate_w: Optional[torch.Tensor], up_w: torch.Tensor, down_w: torch.Tensor,
+                limit: float, alpha: float, shift: float, in_scale: Optional[torch.Tensor] = None,
+                activation: str = "identity") -> torch.Tensor:
     """Every (token, choice) pair through its expert: float32 [T * top, width], row t * top + j the output of expert
     ids[t, j] for token t.  gate_w, up_w [E, ff, width], down_w [E, width, ff].  in_scale (float32 [T, top]): a factor
-    on the expert's input for every pair, applied to the float32 sums of the gate and up products."""
+    on the expert's input for every pair, applied to the float32 sums of the gate and up products.
+    gate_w None: experts without a gate, down(activation(up(x))).  A choice outside 0 .. E - 1 (an expert without
+    tensors) runs nothing, and its row is left unwritten."""
     _need_cuda(x, ids, gate_w, up_w, down_w, in_scale)
+    gated = gate_w is not None
+    if not gated:
+        gate_w = up_w
     if in_scale is not None and (in_scale.dtype != torch.float32 or tuple(in_scale.shape) != tuple(ids.shape) or not in_scale.is_contiguous()):
         raise ValueError("in_scale is a contiguous float32 tensor of the shape of ids")
     _rows2d("x", x)
@@ -876,21 +1038,24 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, gate_w: torch.Tensor, up_w: 
     hidden = torch.empty(n_pairs, ff, dtype=x.dtype, device=x.device)
     y = torch.empty(n_pairs, width, dtype=torch.float32, device=x.device)
     code = _code(x.dtype)
-    check(lib.fmsamd_moe_experts(0, x.data_ptr(), x.stride(0), gate_w.data_ptr(), up_w.data_ptr(), hidden.data_ptr(), code,
+    check(lib.fmsamd_moe_experts(0, x.data_ptr(), x.stride(0), gate_w.data_ptr(), up_w.data_ptr() if gated else None, hidden.data_ptr(), code,
                                  order.data_ptr(), tiles.data_ptr(), max_tiles, tile_rows, top, ff, width, float(limit), float(alpha), float(shift),
-                                 _ptr(in_scale), _stream()))
+                                 _ptr(in_scale), ACTIVATIONS[activation], _stream()))
     check(lib.fmsamd_moe_experts(1, hidden.data_ptr(), hidden.stride(0), down_w.data_ptr(), None, y.data_ptr(), code,
                                  order.data_ptr(), tiles.data_ptr(), max_tiles, tile_rows, top, width, ff, float(limit), float(alpha), float(shift),
-                                 None, _stream()))
+                                 None, 0, _stream()))
     return y
 
 
 def moe_combine(y: torch.Tensor, weights: Optional[torch.Tensor], shared: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor],
-                out_dtype: torch.dtype, top: int = 0) -> torch.Tensor:
+                out_dtype: torch.dtype, top: int = 0, ids: Optional[torch.Tensor] = None, n_experts: int = 0,
+                x_in: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t] = sum_j weights[t, j] * y[t * top + j] (+ sigmoid(shared_gate[t]) * shared[t]) in out_dtype.
     weights None (then `top` says how many rows a token has): the plain sum.
-    shared_gate: a float32 column view [T] (any row stride) of logits, or None for an ungated shared output."""
-    _need_cuda(y, weights, shared, shared_gate)
+    shared_gate: a float32 column view [T] (any row stride) of logits, or None for an ungated shared output.
+    ids [T, top] with n_experts and x_in [T, width] (of out_dtype): a choice of n_experts or more is an identity
+    expert, whose output is the token's row of x_in."""
+    _need_cuda(y, weights, shared, shared_gate, ids, x_in)
     if weights is not None:
         T, top = weights.shape
     elif top <= 0 or y.dim() != 2 or y.shape[0] % top:
@@ -908,9 +1073,15 @@ def moe_combine(y: torch.Tensor, weights: Optional[torch.Tensor], shared: Option
         if shared is None or shared_gate.dtype != torch.float32 or shared_gate.dim() != 1 or shared_gate.shape[0] != T:
             raise ValueError("the shared gate is a float32 [T] view and needs a shared output")
         ldg = shared_gate.stride(0)
+    if ids is not None:
+        _need_i32("ids", ids)
+        if tuple(ids.shape) != (T, top) or x_in is None or x_in.dtype != out_dtype or x_in.dim() != 2 or x_in.stride(1) != 1 \
+                or tuple(x_in.shape) != (T, width):
+            raise ValueError("identity experts need ids [T, top] and the tokens' inputs [T, width] of the output type")
     out = torch.empty(T, width, dtype=out_dtype, device=y.device)
     check(load().fmsamd_moe_combine(y.data_ptr(), _ptr(weights), top, _ptr(shared), _ptr(shared_gate), ldg, out.data_ptr(),
-                                    _code(out_dtype), T, width, _stream()))
+                                    _code(out_dtype), T, width, _ptr(ids), int(n_experts), _ptr(x_in) if ids is not None else None,
+                                    x_in.stride(0) if ids is not None else 0, _stream()))
     return out
 
 

@@ -1,7 +1,7 @@
-from . import attention, block, embedding, experts, feedforward, gated_delta, latent_attention, linear, norm, parallel, position  # noqa: F401  (register the parts)
+from . import attention, block, embedding, experts, feedforward, gated_delta, latent_attention, linear, norm, parallel, position, rglru  # noqa: F401  (register the parts)
 from .attention import LayerCache, MultiHeadAttention
 from .base import BranchOutput, FeedForward, Mixer, NormedRows, ParamSpec, Part, list_parts, make_part, part_attribute, register_part, unregister_part
-from .block import PreNormBlock, ResidualStream, SandwichNormBlock
+from .block import PostNormBlock, PreNormBlock, ResidualStream, SandwichNormBlock
 from .embedding import LinearHead, TokenEmbedding
 from .experts import MLP, ExpertsFeedForward
 from .feedforward import GatedLinearUnit
@@ -10,6 +10,7 @@ from .latent_attention import LatentAttention
 from .linear import Linear
 from .norm import ParameterizedNorm
 from .parallel import ParallelMixers
+from .rglru import RecurrentGatedUnit
 from .position import PositionEncoding, RotaryEncoding, rope_frequencies
 from .spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
 

@@ -13,6 +13,7 @@ from typing import Optional
 
 import torch
 
+from ..cache import StateNeed
 from ..kernels import ops
 from .base import BranchOutput, NormedRows, Part, register_part
 
@@ -43,6 +44,23 @@ class ResidualStream:
         if pending_norm is not None:
             return norm.add_norm(self.resid, pending, act_dtype, rows, branch_norm=pending_norm)
         return norm.add_norm(self.resid, pending, act_dtype, rows)
+
+    def rows(self, act_dtype: torch.dtype, want_rows: bool = True) -> Optional[torch.Tensor]:
+        """The stream itself, not normed, with what is pending added: in the activation type if `want_rows` (in a
+        float32 model the stream's own tensor), else nothing.  For blocks whose branches read the stream as it is."""
+        self.prepared = None
+        pending, self.pending = self.pending, None
+        pending_norm, self.pending_norm = self.pending_norm, None
+        if pending is not None and pending_norm is None:
+            raise NotImplementedError("a branch without a norm of its own is added by the norm that reads the stream next")
+        copy_wanted = want_rows and act_dtype != torch.float32
+        if pending is not None:
+            out = pending_norm.join(self.resid, pending, pending.dtype, copy_wanted)
+        else:
+            out = ops.cast(self.resid, act_dtype) if copy_wanted else None
+        if not want_rows:
+            return None
+        return out if copy_wanted else self.resid
 
     def add_branch(self, out, next_norm: Optional[Part] = None, post_norm: Optional[Part] = None) -> None:
         """Takes a branch's output: a tensor (added when the stream is next read) or a BranchOutput.  post_norm: the
@@ -132,5 +150,50 @@ class SandwichNormBlock(Part):
             stream.add_branch(self.feed_forward.forward(h), post_norm=self.norm2b)
 
 
+class PostNormBlock(Part):
+    """A block whose norms sit behind its branches only: h = x + norm1(mixer(x')); y = h + norm2(ff(h)).  The branches read
+    the stream itself.  With `input_taps` the mixer reads x' = x + conv(x), a causal convolution over time on every
+    channel of the stream (weight [width, taps], no bias, the last column the token's own); the stream's last
+    taps - 1 rows are then part of a sequence's state.  The feed-forward may be absent (None).  The norm behind a branch
+    and the residual sum are one kernel, which also leaves what the next branch reads."""
+
+    norm_arguments = ("norm1", "norm2")
+
+    def __init__(self, mixer: Part, feed_forward: Optional[Part], norm1: Part, norm2: Part, width: int = 0, input_taps: int = 0,
+                 names=("norm1", "mix", "norm2", "mlp", "canon1")):
+        super().__init__()
+        self.mixer = self.add_child(names[1], mixer)
+        self.norm1 = self.add_child(names[0], norm1)
+        self.feed_forward = feed_forward
+        if feed_forward is not None:
+            self.norm2 = self.add_child(names[2], norm2)
+            self.add_child(names[3], feed_forward)
+        self.input_taps = int(input_taps)
+        self.width = int(width)
+        self._conv_name = names[4]
+        if self.input_taps:
+            if not 1 <= self.input_taps <= ops.CONV_MAX_TAPS or self.width <= 0:
+                raise ValueError(f"an input convolution of {input_taps} taps (1 to {ops.CONV_MAX_TAPS}) over {width} channels")
+            self.declare(names[4], (self.width, self.input_taps))
+
+    def state_need(self) -> Optional[StateNeed]:
+        """The stream's last taps - 1 rows of every sequence (float32), under a name that no mixer's state has."""
+        if self.input_taps > 1:
+            return StateNeed((("block.conv", (self.input_taps - 1, self.width), "float32"),))
+        return None
+
+    def forward(self, stream: ResidualStream, batch, cache, act_dtype: torch.dtype, next_norm: Optional[Part] = None) -> None:
+        if self.input_taps:
+            x = stream.rows(torch.float32)
+            h = ops.short_conv(x, 0, self.width, self.w[self._conv_name], None, cache.state.get("block.conv"), batch.seq_of_token,
+                               batch.slot_ids, act_dtype, add_input=True)
+        else:
+            h = stream.rows(act_dtype)
+        stream.add_branch(self.mixer.forward(h, batch, cache), post_norm=self.norm1)
+        if self.feed_forward is not None:
+            stream.add_branch(self.feed_forward.forward(stream.rows(act_dtype)), post_norm=self.norm2)
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "post_norm", PostNormBlock)
 register_part("block", "sandwich_norm", SandwichNormBlock)

@@ -7,7 +7,8 @@ space, runs attention as one shared kv head over the cached rows, and takes the 
 prompts, portions of prompts and single tokens run the same kernels over the same cache, so how a sequence is cut
 into steps changes nothing beyond rounding.
 
-Options, all constructor arguments: queries through a latent of their own with an RMS norm (q_rank), a sink logit
+Options, all constructor arguments: queries through a latent of their own with an RMS norm (q_rank; 0: the queries
+are one projection of the mixer's input), no rotated part at all (rot_dim 0, attention without positions), a sink logit
 per head in the softmax's denominator, a sigmoid gate per head on the output (read from the mixer's input), a
 window, and `owns_kv=False` for a layer that reads the latent and key part that another layer cached (it then has
 no down-projection for them; its Uk, Uv, queries and everything else are its own).
@@ -45,7 +46,7 @@ class LatentAttention(Mixer):
         position_encoder: Optional[PositionEncoding] = None,
     ):
         super().__init__()
-        if min(nheads, dim, vdim, q_rank, kv_rank) <= 0 or rot_dim < 0 or rot_dim % 2:
+        if min(nheads, dim, vdim, kv_rank) <= 0 or q_rank < 0 or rot_dim < 0 or rot_dim % 2:
             raise ValueError("latent attention needs positive sizes and an even rotated size")
         if rot_dim and position_encoder is None:
             raise ValueError("a rotated key part needs a position encoding")
@@ -53,14 +54,18 @@ class LatentAttention(Mixer):
         self.q_rank, self.kv_rank, self.scale, self.eps = q_rank, kv_rank, float(scale), float(eps)
         self.has_sink, self.has_gate, self.owns_kv, self.window = bool(sink), bool(output_gate), bool(owns_kv), int(window)
         self.position_encoder = position_encoder
-        # one product for everything that reads the mixer's input: [query latent | gate logits | kv latent, shared key part]
-        self.gate_col = q_rank
-        self.kv_col = q_rank + (nheads if output_gate else 0)
+        # one product for everything that reads the mixer's input: [query latent (or the queries themselves) | gate logits |
+        # kv latent, shared key part]
+        self.q_cols = q_rank if q_rank else nheads * (dim + rot_dim)
+        self.gate_col = self.q_cols
+        self.kv_col = self.q_cols + (nheads if output_gate else 0)
         self.down = self.add_child("down", Linear(width, self.kv_col + ((kv_rank + rot_dim) if owns_kv else 0)))
-        self.declare("q_norm.weight", (q_rank,), init="ones", kind="scale")
+        if q_rank:
+            self.declare("q_norm.weight", (q_rank,), init="ones", kind="scale")
         if owns_kv:
             self.declare("kv_norm.weight", (kv_rank,), init="ones", kind="scale")
-        self.uq = self.add_child("uq", Linear(q_rank, nheads * (dim + rot_dim)))
+        if q_rank:
+            self.uq = self.add_child("uq", Linear(q_rank, nheads * (dim + rot_dim)))
         self.declare("uk.weight", (nheads * dim, kv_rank))
         self.declare("uv.weight", (nheads * vdim, kv_rank))
         if sink:
@@ -73,7 +78,7 @@ class LatentAttention(Mixer):
         """The fused down-projection as the tensors it is made of, in the order of its rows (what the model's
         state_dict(fused_weights=False) shows in its place)."""
         H = self.nheads
-        pieces = [("dq", self.q_rank)] + ([("g", H)] if self.has_gate else []) + ([("dkv", self.kv_rank + self.rot_dim)] if self.owns_kv else [])
+        pieces = [("dq" if self.q_rank else "q", self.q_cols)] + ([("g", H)] if self.has_gate else []) + ([("dkv", self.kv_rank + self.rot_dim)] if self.owns_kv else [])
         return {"down": tuple(pieces)}
 
     def kv_need(self) -> Optional[KVNeed]:
@@ -120,8 +125,11 @@ class LatentAttention(Mixer):
                 raise RuntimeError("this layer has no down-projection for keys and values: it must read another layer's cache")
             ops.latent_kv_write(down, self.kv_col, R, P, self.w["kv_norm.weight"], self.eps, batch.positions, batch.seq_of_token,
                                 table, cos, sin, cache.keys, cache.values)
-        cq = ops.rms_norm_cols(down, 0, self.q_rank, self.w["q_norm.weight"], self.eps, x.dtype)
-        q = self.uq.forward(cq)
+        if self.q_rank:
+            cq = ops.rms_norm_cols(down, 0, self.q_rank, self.w["q_norm.weight"], self.eps, x.dtype)
+            q = self.uq.forward(cq)
+        else:
+            q = down[:, : self.q_cols] if down.dtype == x.dtype else ops.cast_cols(down, 0, self.q_cols, x.dtype)
         qa = torch.empty(T, H * (R + P), dtype=x.dtype, device=x.device)
         if P:
             ops.latent_q_rotate(q, qa, H, D, P, R, batch.positions, cos, sin)
