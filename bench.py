@@ -22,6 +22,12 @@ flops would take at what this GPU delivers (`x_roofline`: 1 is the roofline).
 
 is the same comparison for Defapel (windowed attention beside a gated delta rule, a delta rule with a decay per channel,
 experts weighted on their input) beside Llama of the same width, depth and heads.
+
+    python bench.py --sidalorn [--layers N]
+
+is the same comparison for Sidalorn (attention without positions over a latent, a real-gated recurrent block, norms in
+groups behind the branches, experts routed in groups) beside Zodolorn, the closest model of the library (attention over
+a latent, experts), with the same width, depth, heads, latent and expert sizes.
 """
 
 import argparse
@@ -66,6 +72,7 @@ def main() -> int:
     ap.add_argument("--zodolorn", action="store_true",
                     help="another workload: Zodolorn beside Llama at equal layer sizes, with every kernel class's distance from its roofline")
     ap.add_argument("--defapel", action="store_true", help="another workload: Defapel beside Llama at equal layer sizes, likewise")
+    ap.add_argument("--sidalorn", action="store_true", help="another workload: Sidalorn beside Zodolorn at equal layer sizes, likewise")
     args = ap.parse_args()
     if args.seq_len is not None:
         args.prompt_min = args.prompt_max = args.seq_len
@@ -77,8 +84,8 @@ def main() -> int:
         print(f"bench.py measures one GPU: this library runs on a single MI355X, --gpus {args.gpus} is not supported")
         return 2
 
-    if args.zodolorn or args.defapel:
-        return design_comparison(args, "zodolorn" if args.zodolorn else "defapel")
+    if args.zodolorn or args.defapel or args.sidalorn:
+        return design_comparison(args, "zodolorn" if args.zodolorn else ("defapel" if args.defapel else "sidalorn"))
 
     import torch
 
@@ -320,6 +327,14 @@ DEFAPEL_SIZES = [
 ]
 
 
+# (name, width, layer pattern, heads, [dim, vdim, kv_rank], recurrent channels, blocks, dense ff, experts, identity experts, top,
+#  expert ff, shared ff, groups, groups kept, norm groups, vocabulary)
+SIDALORN_SIZES = [
+    ("w2048", 2048, "aar", 16, (128, 128, 512), 2560, 10, 8192, 28, 4, 4, 1024, 2048, 4, 2, 4, 32768),
+    ("w4096", 4096, "aar", 32, (128, 128, 512), 4096, 16, 12288, 60, 4, 6, 1536, 3072, 8, 4, 8, 32768),
+]
+
+
 def design_comparison(args, design) -> int:
     import torch
 
@@ -361,6 +376,16 @@ def design_comparison(args, design) -> int:
         if name == "latent_attention":  # one row of rank + rot a key, and the latent once more as values
             H, R, P = a[6], a[7], a[8]
             return 2 * state["keys_loaded"] * (2 * R + P) + nbytes(a[0]) + 2 * a[0].shape[0] * H * R, 2.0 * state["keys_read"] * H * (2 * R + P)
+        if name == "rglru_gates":  # two block-diagonal products on the float32 vector units, priced like the delta rule's passes
+            u, ra = a[0], a[1]
+            vector_flops = 4.0 * u.shape[0] * ra.numel()
+            return nbytes(u, ra, a[3]) + 2 * u.numel() * 4, vector_flops * mfma_flops / PEAK_FLOPS["fp32"]
+        if name == "rglru_scan":  # a, b and the other branch read once, the result written once
+            return nbytes(a[0], a[1]) + a[0].numel() * 4 + nbytes(out), 0.0
+        if name == "moe_experts" and a[2] is None:  # experts without a gate
+            x, ids, _, u, d = a[:5]
+            used = min(u.shape[0], ids.numel())
+            return used * (nbytes(u, d) // u.shape[0]) + ids.numel() * (2 * x.shape[1] * x.element_size() + 4 * x.shape[1]), 4.0 * ids.numel() * u.shape[1] * u.shape[2]
         if name == "moe_experts":
             x, ids, g, u, d = a[:5]
             used = min(g.shape[0], ids.numel())  # experts whose weights are read at least once
@@ -371,10 +396,12 @@ def design_comparison(args, design) -> int:
     watched = ["linear", "gated_linear", "linear_into_stream", "headwise_linear", "attention", "latent_attention", "moe_experts",
                "moe_route", "moe_combine", "add_norm", "norm_add_norm", "rms_norm_cols", "rope_kv_write", "qkv_rope_write",
                "latent_kv_write", "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed",
-               "delta_rule", "delta_prepare", "gated_head_norm", "qk_projection_norm", "gate_mul", "scale_", "cast", "cast_cols"]
+               "delta_rule", "delta_prepare", "gated_head_norm", "qk_projection_norm", "gate_mul", "scale_", "cast", "cast_cols",
+               "rglru_gates", "rglru_scan", "short_conv", "group_norm_chain", "poly_norm", "moe_route_grouped"]
     small = {"moe_route", "moe_combine", "add_norm", "norm_add_norm", "rms_norm_cols", "rope_kv_write", "latent_kv_write",
              "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed", "delta_prepare", "gated_head_norm",
-             "qk_projection_norm", "gate_mul", "scale_", "cast", "cast_cols"}
+             "qk_projection_norm", "gate_mul", "scale_", "cast", "cast_cols", "short_conv", "group_norm_chain", "poly_norm",
+             "moe_route_grouped"}
 
     def classes_of_a_step(run):
         """{class: (ms, ms at the roofline)} of the kernels of `run()`, by events around every call into the library."""
@@ -471,7 +498,7 @@ def design_comparison(args, design) -> int:
             torch.cuda.empty_cache()
         return out
 
-    record = {"workload": f"{design} beside llama at equal layer sizes", "layers": layers, "dtype": "bf16",
+    record = {"workload": f"{design} beside {'zodolorn' if design == 'sidalorn' else 'llama'} at equal layer sizes", "layers": layers, "dtype": "bf16",
               "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
               "peak_measured": {"read_gbs": round(read_bps / 1e9, 1), "mfma_tflops": round(mfma_flops / 1e12, 1)}, "sizes": {}}
     if design == "defapel":
@@ -498,6 +525,38 @@ def design_comparison(args, design) -> int:
                                                                    experts=experts, top=top, expert_ff=expert_ff, vocab=vocab), **mine),
                                      "llama": dict(config=dict(width=width, heads=heads, kvheads=kv, head_dim=width // heads, hidden=hidden,
                                                                vocab=vocab), **theirs)}
+        print(json.dumps(record))
+        return 0
+    if design == "sidalorn":
+        from fms_amd.architectures.sidalorn import make_config as make_sidalorn
+
+        for (name, width, pattern, heads, (dim, vdim, kv_rank), channels, blocks, dense_ff, experts, identity, top, expert_ff, shared_ff,
+             groups, keep, norm_groups, vocab) in SIDALORN_SIZES:
+            pattern = (pattern * layers)[:layers]
+            config = make_sidalorn(width=width, vocab=vocab, pattern=pattern, heads=heads, dim=dim, vdim=vdim, kv_rank=kv_rank,
+                                   recurrent_width=channels, blocks=blocks, dense_ff=dense_ff, experts=experts, top=top, expert_ff=expert_ff,
+                                   identity=identity, shared_ff=shared_ff, group_count=groups, group_keep=keep, route_scale=2.0,
+                                   norm_groups=norm_groups, max_positions=context)
+            model = fms_amd.from_config(config, "sidalorn", data_type="bf16", random_seed=args.seed)
+            mine = measure(model, vocab)
+            del model
+            torch.cuda.empty_cache()
+            # Zodolorn of the same width, depth, heads, latent and feed-forward sizes (its keys also carry a rotated part,
+            # its queries pass a latent of their own, its experts have gates)
+            other = make_config(width=width, vocab=vocab, nlayers=layers, heads=heads, dim=dim, rot_dim=64, vdim=vdim, q_rank=3 * kv_rank // 2,
+                                kv_rank=kv_rank, dense_ff=dense_ff, experts=experts + identity, top=top, expert_ff=expert_ff,
+                                shared_ff=shared_ff, max_positions=context)
+            zodolorn = fms_amd.from_config(other, "zodolorn", data_type="bf16", random_seed=args.seed)
+            theirs = measure(zodolorn, vocab)
+            del zodolorn
+            torch.cuda.empty_cache()
+            record["sizes"][name] = {"sidalorn": dict(config=dict(width=width, pattern=pattern, heads=heads, dim=dim, vdim=vdim, kv_rank=kv_rank,
+                                                                    recurrent_width=channels, blocks=blocks, dense_ff=dense_ff, experts=experts,
+                                                                    identity=identity, top=top, expert_ff=expert_ff, shared_ff=shared_ff,
+                                                                    groups=groups, keep=keep, norm_groups=norm_groups, vocab=vocab), **mine),
+                                     "zodolorn": dict(config=dict(width=width, heads=heads, dim=dim, rot_dim=64, vdim=vdim, q_rank=3 * kv_rank // 2,
+                                                                    kv_rank=kv_rank, dense_ff=dense_ff, experts=experts + identity, top=top,
+                                                                    expert_ff=expert_ff, shared_ff=shared_ff, vocab=vocab), **theirs)}
         print(json.dumps(record))
         return 0
     for name, width, heads, (dim, rot, vdim, q_rank, kv_rank), dense_ff, experts, top, expert_ff, shared_ff, vocab in ZODOLORN_SIZES:

@@ -1,0 +1,853 @@
+"""Sidalorn on the GPU against the plain implementation (plain_sidalorn.py): every mechanism alone, then the engine
+whole / token by token / in portions / in ragged batches with reused slots / through graphs and the generation loop,
+in float32 and bfloat16, at sizes that differ from one another in everything.
+
+bfloat16 is judged like the other models of this folder (gpu_checks): the plain implementation run with bfloat16
+storage shows what that type costs at every position, and the engine may be a small multiple of that off."""
+
+import json
+import math
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import plain_sidalorn as S  # noqa: E402
+from gpu_checks import Expected  # noqa: E402
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEV = "cuda"
+DTYPES = ["float32", "bfloat16"]
+# bfloat16: at every position the engine may be BF16_MARGIN times as far off as the plain implementation with bfloat16
+# storage is there (or as it typically is), and on average BF16_MEAN_MARGIN times.  The engine rounds in other places
+# than the plain implementation (queries and attention results in the latent space instead of keys and values), and
+# this design's errors have a long tail: the norm behind a branch divides by the branch's own size, so where a branch's
+# output is small (a sink that holds most of a softmax's weight, experts that cancel) its rounding error grows with it.
+# Layer by layer the engine's median and largest error over a sequence are those of the plain implementation with
+# bfloat16 storage (within a tenth); at single positions the two draw differently from that tail: the plain
+# implementation's own worst position is up to 3.8 times its 90th percentile in the sequences of this file, the
+# engine's up to 4.6 times.  What the tests are there to find is far larger: a lost key or a lost recurrent state moves
+# the logits by 50 times the typical error.
+BF16_MARGIN = 5.0
+BF16_MEAN_MARGIN = 1.5
+# A router's choice is "close" when a change of the router's logits by about this much turns it (the plain
+# implementation's measure: the lead of the last chosen output, or of the last kept group, over the best one left out,
+# in units of the scores involved): bfloat16 rounding can do that, the token then runs other experts, and its logits are
+# no test of arithmetic.  Such positions are left out of bfloat16 comparisons.
+CLOSE_CALL = 0.15
+
+
+def attention(heads, dim, vdim, kv_rank, scale):
+    return {"type": "latent_attention", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": kv_rank, "scale": scale}}
+
+
+def recurrent(width, blocks, conv):
+    return {"type": "rglru", "mixer": {"width": width, "blocks": blocks, "conv": conv}}
+
+
+def moe(experts, identity, top, ff, count=1, keep=1, scale=1.0, shared=0):
+    out = {"kind": "moe", "expert": {"ff": ff},
+           "router": {"experts": experts, "identity": identity, "top": top, "scale": scale, "groups": {"count": count, "keep": keep}}}
+    if shared:
+        out["shared"] = {"ff": shared}
+    return out
+
+
+def layer(mixer, mlp):
+    return dict(mixer, mlp=mlp)
+
+
+CONFIGS = {
+    # a recurrent layer first; attention whose key, value and latent sizes all differ and whose heads do not fill the
+    # width; a layer without a feed-forward; experts in groups with identity experts and a shared one; identity experts
+    # that outnumber the others; taps of the stream's convolution and of the recurrent block's differ
+    "A": dict(vocab=300, width=128, norm={"eps": 1e-5, "groups": 2}, canon={"taps": 3}, max_positions=1024, layers=[
+        layer(recurrent(96, 3, 4), {"kind": "dense", "ff": 160}),
+        layer(attention(4, 16, 24, 40, 0.2), moe(6, 3, 3, 48, count=3, keep=2, scale=1.5, shared=64)),
+        layer(attention(2, 32, 8, 24, 0.3), None),
+        layer(recurrent(64, 1, 2), moe(2, 4, 2, 40, count=2, keep=1, scale=0.5)),
+        layer(attention(4, 16, 24, 40, 0.25), {"kind": "dense", "ff": 96}),
+    ]),
+    # sizes that are no multiples of 8 (rows that the matrix instructions cannot load); one norm group; a stream
+    # convolution of one tap (no state) and of the recurrent block's; one expert per token; no groups, no identity
+    # experts, no shared expert in one layer, all experts chosen in another
+    "B": dict(vocab=257, width=100, norm={"eps": 1e-6, "groups": 1}, canon={"taps": 1}, max_positions=1024, layers=[
+        layer(attention(3, 12, 20, 28, 0.31), moe(5, 0, 1, 36)),
+        layer(recurrent(60, 5, 1), {"kind": "dense", "ff": 60}),
+        layer(attention(2, 20, 8, 36, 0.25), moe(3, 1, 4, 44, count=2, keep=2, scale=3.0, shared=52)),
+    ]),
+    # sizes at which bfloat16 runs the matrix-instruction kernels throughout; five taps; only identity experts beside a
+    # shared one in the last layer
+    "C": dict(vocab=512, width=256, norm={"eps": 1e-6, "groups": 8}, canon={"taps": 5}, max_positions=2048, layers=[
+        layer(attention(8, 64, 48, 128, 0.1), {"kind": "dense", "ff": 512}),
+        layer(recurrent(384, 3, 4), moe(8, 4, 3, 128, count=4, keep=2, scale=2.5, shared=128)),
+        layer(attention(4, 128, 64, 64, 0.08), moe(0, 4, 2, 0, count=2, keep=1, scale=1.0, shared=256)),
+    ]),
+}
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import fms_amd
+    from fms_amd.kernels import load
+
+    load()
+    return fms_amd
+
+
+def write_folder(lib, folder, cfg_kw, seed, sharp=1.0):
+    """A model folder with random weights in which every number matters: sinks of the size of the scores, noisy norm
+    scales, routers with clear choices and corrections of the size of the scores (some negative), biases, decays from
+    fast to slow, stream convolutions that weigh as much as the token itself."""
+    from fms_amd.weights import write_safetensors
+
+    lib.write_model_folder(folder, lib.SidalornConfig(**cfg_kw), seed=seed, architecture="sidalorn", std=0.08, norm_std=0.2)
+    cfg, tensors = S.load_model_folder(folder)
+    gen = torch.Generator().manual_seed(seed)
+
+    def noise(t, std, mean=0.0):
+        return mean + std * torch.randn(t.shape, generator=gen, dtype=torch.float64)
+
+    for k in list(tensors):
+        t = tensors[k]
+        if k.endswith(".mix.sink"):
+            tensors[k] = noise(t, 1.5)
+        elif k.endswith(".mlp.router"):
+            tensors[k] = t * 4
+        elif k.endswith(".mlp.correction"):
+            tensors[k] = noise(t, 0.6 / t.shape[0])
+        elif k.endswith(".mix.lam"):
+            tensors[k] = noise(t, 2.0, -3.0)
+        elif k.endswith((".ra.b", ".ri.b", ".x.b", ".y.b", ".conv.b")):
+            tensors[k] = noise(t, 0.5)
+        elif k.endswith((".mix.ra", ".mix.ri", ".mix.conv")):
+            tensors[k] = t * 4
+        elif k.endswith(".canon1"):
+            tensors[k] = noise(t, 0.5)
+        elif k.endswith(".mlp.act"):
+            tensors[k] = torch.tensor([0.7, 0.4, 0.25, 0.1], dtype=torch.float64) + noise(t, 0.1)
+        elif sharp != 1.0 and k == "l0.mix.q":
+            tensors[k] = t * sharp  # the first layer's queries: its scores are formed from the embedding, which is small
+    tensors = {k: v.to(torch.bfloat16) for k, v in tensors.items()}
+    write_safetensors(os.path.join(folder, "model.safetensors"), [(k, tuple(v.shape), v.dtype) for k, v in tensors.items()],
+                      lambda name: tensors[name])
+    return folder
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory, lib):
+    return {name: write_folder(lib, str(tmp_path_factory.mktemp(f"sidalorn_{name}")), kw, 3 + i) for i, (name, kw) in enumerate(CONFIGS.items())}
+
+
+_models, _plain, _expected = {}, {}, {}
+
+
+def get(lib, folders, name, dtype):
+    if (name, dtype) not in _models:
+        _models[(name, dtype)] = lib.get_model("hf_pretrained", model_path=folders[name], data_type=dtype)
+    return _models[(name, dtype)]
+
+
+def plain(folders, name):
+    if name not in _plain:
+        _plain[name] = S.load_model_folder(folders[name])
+    return _plain[name]
+
+
+def tokens_for(vocab, n, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def expect(cfg, weights, ids, dtype) -> Expected:
+    """Exact logits; for bfloat16 also the plain implementation's own error with bfloat16 storage, set to infinity at
+    the positions where a router's choice is close (they are not compared), and its 90th percentile over the rest."""
+    margins = []
+    exact = S.forward(cfg, weights, ids, margins=margins)
+    if dtype == "float32":
+        return Expected(exact)
+    rounded = S.forward(cfg, weights, ids, rounding="bfloat16")
+    error = (rounded - exact).abs().amax(dim=-1)
+    close = torch.zeros(len(ids), dtype=torch.bool)
+    for gap in margins:
+        close |= gap < CLOSE_CALL
+    assert float(close.float().mean()) < 0.5, "most positions have close router calls: the test would compare little"
+    typical = torch.quantile(error[~close], 0.9).expand_as(error)
+    return Expected(exact, torch.where(close, torch.full_like(error, float("inf")), error), typical)
+
+
+def expected_for(folders, name, n, seed, dtype):
+    key = (name, n, seed, dtype)
+    if key not in _expected:
+        cfg, weights = plain(folders, name)
+        ids = tokens_for(cfg["vocab"], n, seed)
+        _expected[key] = (ids, expect(cfg, weights, ids, dtype))
+    return _expected[key]
+
+
+def judge(got, want, dtype):
+    got = got.float().cpu()
+    assert got.shape == want.shape, f"{tuple(got.shape)} logits, {tuple(want.shape)} expected"
+    if dtype == "float32":
+        torch.testing.assert_close(got, want.logits, atol=2e-4, rtol=1e-3)
+        return
+    error = (got - want.logits).abs().amax(dim=-1).flatten()
+    ref, typical = want.ref_error.flatten(), want.typical.flatten()
+    compared = torch.isfinite(ref)
+    allowed = BF16_MARGIN * torch.maximum(ref, typical)
+    worst = int(torch.argmax(torch.where(compared, error / allowed, torch.zeros_like(error))))
+    assert bool((error[compared] <= allowed[compared]).all()), (
+        f"bfloat16 logits are {float(error[worst]):.4g} off at row {worst}; the plain implementation with bfloat16 storage is "
+        f"{float(ref[worst]):.4g} off there and typically {float(typical[worst]):.4g} (allowed: {BF16_MARGIN} times the larger)")
+    if int(compared.sum()) >= 32:
+        assert float(error[compared].mean()) <= BF16_MEAN_MARGIN * float(ref[compared].mean()), (
+            f"bfloat16 logits are {float(error[compared].mean()):.4g} off on average, the plain implementation with bfloat16 "
+            f"storage {float(ref[compared].mean()):.4g}")
+
+
+def _i32(values):
+    return torch.tensor(values, dtype=torch.int32, device=DEV)
+
+
+# ---- mechanisms alone ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [(40, 1, 1), (192, 4, 2), (1000, 5, 8), (3000, 3, 1), (4096, 8, 4), (36, 36, 6)])
+def test_norm_in_groups_behind_a_branch_the_sum_and_what_is_read_next(lib, dtype, sizes):
+    from fms_amd.kernels import ops
+
+    width, bgroups, groups = sizes
+    gen = torch.Generator().manual_seed(width)
+    resid = torch.randn(7, width, generator=gen) * 3
+    branch = (torch.randn(7, width, generator=gen) * 5).to(dtype)
+    branch[:, : width // bgroups] *= 20  # one group far larger than the others: a norm over the whole row would show
+    wb, w = 1 + 0.3 * torch.randn(width, generator=gen), 1 + 0.3 * torch.randn(width, generator=gen)
+    total = resid + S.norm_in_groups(branch.double(), wb.double(), bgroups, 1e-3).float()
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=1e-2)
+    # the sum alone; the sum and the stream in the activation type; the sum and the next norm
+    r = resid.to(DEV).clone()
+    assert ops.group_norm_chain(r, branch.to(DEV), wb.to(DEV), bgroups, 1e-3, dtype, ops.CHAIN_NONE) is None
+    torch.testing.assert_close(r.cpu(), total, atol=1e-5, rtol=1e-5)
+    r = resid.to(DEV).clone()
+    out = ops.group_norm_chain(r, branch.to(DEV), wb.to(DEV), bgroups, 1e-3, dtype, ops.CHAIN_CAST)
+    torch.testing.assert_close(r.cpu(), total, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(out.float().cpu(), total, **tol)
+    want = S.norm_in_groups(total.double(), w.double(), groups, 1e-5).float()
+    r = resid.to(DEV).clone()
+    out = ops.group_norm_chain(r, branch.to(DEV), wb.to(DEV), bgroups, 1e-3, dtype, ops.CHAIN_NORM, w.to(DEV), groups, 1e-5)
+    torch.testing.assert_close(r.cpu(), total, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(out.float().cpu(), want, **tol)
+    # chosen rows only (the final norm of a step): the stream stays as it was
+    r2 = resid.to(DEV).clone()
+    out2 = ops.group_norm_chain(r2, branch.to(DEV), wb.to(DEV), bgroups, 1e-3, dtype, ops.CHAIN_NORM, w.to(DEV), groups, 1e-5, rows=_i32([5, 0, 5]))
+    torch.testing.assert_close(out2.float().cpu(), want[[5, 0, 5]], **tol)
+    torch.testing.assert_close(r2.cpu(), resid)
+    # nothing pending: the norm of the stream as it is
+    r3 = total.to(DEV).clone()
+    out3 = ops.group_norm_chain(r3, None, None, 0, 0.0, dtype, ops.CHAIN_NORM, w.to(DEV), groups, 1e-5)
+    torch.testing.assert_close(out3.float().cpu(), want, **tol)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [(1, 24, False), (2, 100, True), (4, 128, True), (5, 36, False), (8, 260, True)])
+def test_convolution_over_time_in_steps_of_any_cut(lib, out_dtype, sizes):
+    """Three sequences in slots that lie apart, fed in ragged steps (whole, portions down to one token, a sequence that
+    joins later into a slot that was used before): every output equals the convolution of the whole sequence."""
+    from fms_amd.kernels import ops
+
+    taps, C, add_input = sizes
+    gen = torch.Generator().manual_seed(taps * 100 + C)
+    lens = [23, 9, 14]
+    xs = [torch.randn(n, C + 5, generator=gen) for n in lens]  # the channels start at column 3 of wider rows
+    w = torch.randn(C, taps, generator=gen)
+    bias = None if add_input else torch.randn(C, generator=gen)
+    want = [S.convolution_over_time(x[:, 3 : 3 + C].double(), w.double(), None if bias is None else bias.double()).float()
+            + (x[:, 3 : 3 + C] if add_input else 0) for x in xs]
+    state = torch.full((6, max(taps - 1, 1), C), 9.0, device=DEV) if taps > 1 else None  # slots hold rubbish until handed out
+    slots = [4, 1, 4]  # the third sequence takes the first one's slot when that has ended
+    schedule = [  # (sequence, tokens) of every step
+        [(0, 5), (1, 1)], [(0, 1), (1, 1)], [(0, 2), (1, 7)], [(0, 15)], [(2, 1)], [(2, 1)], [(2, 12)],
+    ]
+    got = [[] for _ in lens]
+    at = [0, 0, 0]
+    started = set()
+    for step in schedule:
+        rows, seq_of_token, slot_ids = [], [], []
+        for j, (s, n) in enumerate(step):
+            if s not in started:
+                started.add(s)
+                if state is not None:
+                    state[slots[s]].zero_()
+            rows.append(xs[s][at[s] : at[s] + n])
+            seq_of_token += [j] * n
+            slot_ids.append(slots[s])
+        x = torch.cat(rows).to(DEV)
+        out = ops.short_conv(x, 3, C, w.to(DEV), None if bias is None else bias.to(DEV), state, _i32(seq_of_token), _i32(slot_ids),
+                             out_dtype, add_input=add_input)
+        o = 0
+        for s, n in step:
+            got[s].append(out[o : o + n].float().cpu())
+            o += n
+            at[s] += n
+    tol = dict(atol=1e-5, rtol=1e-5) if out_dtype == torch.float32 else dict(atol=3e-2, rtol=1e-2)
+    for s in range(3):
+        assert at[s] == lens[s]
+        torch.testing.assert_close(torch.cat(got[s]), want[s], **tol)
+    if state is not None:  # what a sequence leaves behind: its last taps - 1 inputs, the newest last
+        torch.testing.assert_close(state[1].cpu(), xs[1][-(taps - 1):, 3 : 3 + C])
+        assert float((state[0] - 9.0).abs().max()) == 0.0  # other slots are not touched
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [(12, 3, 5), (60, 5, 19), (128, 1, 8), (384, 3, 33), (64, 64, 7), (1024, 2, 3)])
+def test_gates_of_the_recurrence(lib, wdtype, sizes):
+    from fms_amd.kernels import ops
+
+    C, blocks, T = sizes
+    n = C // blocks
+    gen = torch.Generator().manual_seed(C + T)
+    u = torch.randn(T, C, generator=gen)
+    w = {"ra": (torch.randn(blocks, n, n, generator=gen) * 2 / math.sqrt(n)).to(wdtype), "ri": (torch.randn(blocks, n, n, generator=gen) * 2 / math.sqrt(n)).to(wdtype),
+         "ra.b": torch.randn(blocks, n, generator=gen), "ri.b": torch.randn(blocks, n, generator=gen), "lam": torch.randn(C, generator=gen) * 3 - 2}
+    a_want, b_want = S.recurrence_gates(u.double(), {k: v.double() for k, v in w.items()}, {"blocks": blocks})
+    a, b = ops.rglru_gates(u.to(DEV), w["ra"].transpose(1, 2).contiguous().to(DEV), w["ra.b"].reshape(-1).to(DEV),
+                           w["ri"].transpose(1, 2).contiguous().to(DEV), w["ri.b"].reshape(-1).to(DEV), w["lam"].to(DEV), 8.0,
+                           _i32([0] * T))
+    torch.testing.assert_close(a.cpu(), a_want.float(), atol=2e-6, rtol=2e-5)
+    torch.testing.assert_close(b.cpu(), b_want.float(), atol=2e-6, rtol=5e-5)
+    # slow channels: a close to one keeps its distance from one (sqrt(1 - a^2) is formed without cancellation)
+    slow = a_want > 0.999
+    if bool(slow.any()):
+        torch.testing.assert_close(b.cpu()[slow], b_want.float()[slow], atol=1e-7, rtol=1e-4)
+    # another constant in the decay
+    a5, _ = ops.rglru_gates(u.to(DEV), w["ra"].transpose(1, 2).contiguous().to(DEV), w["ra.b"].reshape(-1).to(DEV),
+                            w["ri"].transpose(1, 2).contiguous().to(DEV), w["ri.b"].reshape(-1).to(DEV), w["lam"].to(DEV), 5.0, _i32([0] * T))
+    torch.testing.assert_close(a5.cpu(), a_want.float() ** (5.0 / 8.0), atol=2e-6, rtol=5e-5)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("C", [12, 64, 300, 1024])
+def test_recurrence_in_steps_of_any_cut(lib, out_dtype, C):
+    """Two sequences in ragged steps, from zero state, one decay close to one: the state after 600 tokens still holds
+    the first token's input, and every output equals the recurrence over the whole sequence."""
+    from fms_amd.kernels import ops
+
+    gen = torch.Generator().manual_seed(C)
+    lens = [600, 77]
+    a = [torch.rand(n, C, generator=gen) for n in lens]
+    a[0][:, 0] = 0.9999
+    b = [torch.randn(n, C, generator=gen) for n in lens]
+    b[0][0, 0] = 200.0
+    y = [torch.randn(n, C + 4, generator=gen) for n in lens]  # the other branch, inside wider rows
+    want = [S.linear_recurrence(a[s].double(), b[s].double()).float() * S.gelu_tanh(y[s][:, 2 : 2 + C].double()).float() for s in range(2)]
+    state = torch.full((5, C), 3.0, device=DEV)
+    slots = [3, 0]
+    state[3].zero_()
+    state[0].zero_()
+    cuts = {0: [1, 1, 2, 60, 64, 65, 300, 1, 106], 1: [70, 1, 1, 1, 2, 1, 1]}
+    assert sum(cuts[0]) == 600 and sum(cuts[1]) == 77
+    got = [[], []]
+    at = [0, 0]
+    for i in range(len(cuts[0])):
+        seqs = [0] + ([1] if i < len(cuts[1]) else [])
+        ns = [cuts[s][i] for s in seqs]
+        starts = [0]
+        for n in ns:
+            starts.append(starts[-1] + n)
+        seq_of_token = [j for j, n in enumerate(ns) for _ in range(n)]
+        cat = lambda parts: torch.cat([parts[s][at[s] : at[s] + n] for s, n in zip(seqs, ns)]).contiguous().to(DEV)  # noqa: E731
+        yy = cat(y)
+        out = ops.rglru_scan(cat(a), cat(b), yy[:, 2 : 2 + C], "gelu-tanh", state, _i32(starts), _i32(seq_of_token), _i32([slots[s] for s in seqs]),
+                             len(seqs), out_dtype)
+        for j, (s, n) in enumerate(zip(seqs, ns)):
+            got[s].append(out[starts[j] : starts[j + 1]].float().cpu())
+            at[s] += n
+    tol = dict(atol=2e-5, rtol=2e-5) if out_dtype == torch.float32 else dict(atol=3e-2, rtol=1e-2)
+    for s in range(2):
+        torch.testing.assert_close(torch.cat(got[s]), want[s], **tol)
+    final = S.linear_recurrence(a[0].double(), b[0].double())[-1].float()
+    torch.testing.assert_close(state[3].cpu(), final, atol=2e-5, rtol=2e-5)
+    assert float(final[0]) > 100.0 and float((state[1] - 3.0).abs().max()) == 0.0  # the first token is still there; other slots untouched
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n", [20, 160, 1001, 5000])
+def test_polynorm(lib, out_dtype, n):
+    from fms_amd.kernels import ops
+
+    z = torch.randn(6, n + 3, generator=torch.Generator().manual_seed(n)) * 2
+    z[1] *= 30  # rows of very different sizes: every row has its own three root mean squares
+    z[2] *= 0.01
+    coefficients = (0.7, -0.4, 0.25, 0.1)
+    want = S.poly_norm(z[:, :n].double(), coefficients, 1e-5).float()
+    got = ops.poly_norm(z.to(DEV)[:, :n], coefficients, 1e-5, out_dtype)
+    tol = dict(atol=1e-5, rtol=1e-5) if out_dtype == torch.float32 else dict(atol=2e-2, rtol=1e-2)
+    torch.testing.assert_close(got.float().cpu(), want, **tol)
+
+
+@pytest.mark.parametrize("sizes", [(12, 4, 3, 2, 1), (6, 3, 3, 2, 40), (5, 1, 1, 1, 9), (64, 8, 8, 3, 300), (130, 6, 10, 4, 17), (8, 8, 2, 2, 5), (9, 2, 3, 1, 64)])
+def test_router_in_groups(lib, sizes):
+    """Choice by score plus correction inside the kept groups only, weights from the scores alone.  Corrections of the
+    size of the scores, half of them negative, so that choice scores below zero are chosen before outputs of groups that are shut out."""
+    from fms_amd.kernels import ops
+
+    n, top, groups, keep, T = sizes
+    gen = torch.Generator().manual_seed(n * 7 + T)
+    logits = torch.randn(T, n + 2, generator=gen) * 3  # two more columns that do not belong to the router
+    correction = torch.randn(n, generator=gen) * (1.5 / n) - (1.0 / n)
+    r = {"top": top, "scale": 1.75, "groups": {"count": groups, "keep": keep}}
+    want_ids, want_w = S.route(logits[:, :n].double(), correction.double(), r)
+    ids, weights = ops.moe_route_grouped(logits.to(DEV), n, top, correction.to(DEV), groups, keep, 1.75)
+    assert ids.cpu().tolist() == want_ids
+    torch.testing.assert_close(weights.cpu(), torch.stack(want_w).float(), atol=1e-6, rtol=1e-5)
+    # no correction: the choice is by the scores themselves
+    ids0, _ = ops.moe_route_grouped(logits.to(DEV), n, top, None, groups, keep, 1.0)
+    assert ids0.cpu().tolist() == S.route(logits[:, :n].double(), torch.zeros(n, dtype=torch.float64), dict(r, scale=1.0))[0]
+
+
+def test_router_prefers_a_negative_choice_score_to_a_group_that_is_shut_out(lib):
+    from fms_amd.kernels import ops
+
+    # two groups of two, one kept: group 0 wins by its 0.4; its other output has a choice score of -0.15 and is still
+    # chosen before 0.3 and 0.25 of the group that is shut out (they count as minus infinity, not as zero)
+    logits = torch.log(torch.tensor([[0.4, 0.05, 0.3, 0.25]]))
+    correction = torch.tensor([0.0, -0.2, 0.0, 0.0])
+    ids, weights = ops.moe_route_grouped(logits.to(DEV), 4, 2, correction.to(DEV), 2, 1, 3.0)
+    assert ids.cpu().tolist() == [[0, 1]]
+    torch.testing.assert_close(weights.cpu(), torch.tensor([[0.4, 0.05]]) / 0.45 * 3.0, atol=1e-6, rtol=1e-5)
+    # all groups kept: the same token takes the two largest choice scores
+    ids, _ = ops.moe_route_grouped(logits.to(DEV), 4, 2, correction.to(DEV), 2, 2, 3.0)
+    assert ids.cpu().tolist() == [[0, 2]]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [(6, 3, 3, 48, 128, 50), (5, 0, 1, 36, 100, 7), (2, 4, 2, 40, 128, 40), (8, 4, 3, 128, 256, 300), (0, 4, 2, 0, 64, 9), (3, 1, 4, 44, 100, 21)])
+def test_experts_without_gates_identity_experts_and_their_sum(lib, dtype, sizes):
+    from fms_amd.kernels import ops
+
+    E, identity, top, ff, width, T = sizes
+    gen = torch.Generator().manual_seed(ff + T)
+    x = torch.randn(T, width, generator=gen).to(dtype)
+    up = (torch.randn(max(E, 1), max(ff, 1), width, generator=gen) * 2 / math.sqrt(width)).to(dtype)
+    down = (torch.randn(max(E, 1), width, max(ff, 1), generator=gen) / math.sqrt(max(ff, 1))).to(dtype)
+    ids = torch.stack([torch.randperm(E + identity, generator=gen)[:top] for _ in range(T)]).to(torch.int32)
+    weights = torch.softmax(torch.randn(T, top, generator=gen), -1) * 1.5
+    shared = torch.randn(T, width, generator=gen).to(dtype)
+    if E:
+        y = ops.moe_experts(x.to(DEV), ids.to(DEV), None, up.to(DEV), down.to(DEV), float("inf"), 1.0, 0.0, activation="gelu")
+    else:
+        y = torch.full((T * top, width), float("nan"), device=DEV)  # no row of it may be read
+    out = ops.moe_combine(y, weights.to(DEV), shared.to(DEV), None, dtype, top=top, ids=ids.to(DEV), n_experts=E, x_in=x.to(DEV))
+    want = shared.float().clone()
+    xf = x.float()
+    for t in range(T):
+        for j in range(top):
+            e = int(ids[t, j])
+            if e >= E:
+                want[t] += weights[t, j] * xf[t]
+                continue
+            h = S.gelu_erf(xf[t] @ up[e].float().T)
+            if dtype == torch.bfloat16:
+                h = h.to(dtype).float()
+            want[t] += weights[t, j] * (h @ down[e].float().T)
+    tol = dict(atol=2e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=5e-2, rtol=2e-2)
+    torch.testing.assert_close(out.float().cpu(), want, **tol)
+    assert int((ids >= E).sum()) > 0 or identity == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [(3, 24), (4, 40), (8, 128), (2, 64), (5, 100), (16, 512)])
+def test_attention_without_positions_over_a_latent_cache(lib, dtype, sizes):
+    """No rotated part at all: two sequences whose pages lie mixed in the pool, queries at page borders and far apart,
+    a sink that matters, and one query and one far key scaled so that the far key decides."""
+    from fms_amd.kernels import ops
+
+    H, R = sizes
+    gen = torch.Generator().manual_seed(R)
+    lens = [130, 200]
+    rows = [torch.randn(n, R, generator=gen).to(dtype) for n in lens]
+    far = 3
+    rows[1][far] *= 4
+    cache = torch.zeros(8, 1, 64, R, dtype=dtype, device=DEV)
+    transposed = torch.zeros(8, 1, R, 64, dtype=dtype, device=DEV)
+    pages = [[6, 1, 4], [0, 7, 2, 5]]
+    for s, plist in enumerate(pages):
+        for j in range(lens[s]):
+            cache[plist[j // 64], 0, j % 64] = rows[s][j].to(DEV)
+            transposed[plist[j // 64], 0, :, j % 64] = rows[s][j].to(DEV)
+    table = _i32([pages[0] + [-1], pages[1]])
+    q_pos = [(0, 129)] + [(1, p) for p in (0, 1, 63, 64, 65, 127, 128, 191, 199)]
+    qa = torch.randn(len(q_pos), H, R, generator=gen).to(dtype)
+    qa[-1, 0] = (rows[1][far].float() / rows[1][far].float().norm() * 6).to(dtype)
+    sink = torch.randn(H, generator=gen) * 2
+    scale = 0.3
+    seq, pos = _i32([s for s, _ in q_pos]), _i32([p for _, p in q_pos])
+    wants = []
+    for i, (s, p) in enumerate(q_pos):
+        keys = rows[s][: p + 1].double()
+        score = torch.einsum("hw,jw->hj", qa[i].double(), keys) * scale
+        top = torch.maximum(score.max(-1).values, sink.double())
+        e = torch.exp(score - top[:, None])
+        prob = e / (e.sum(-1) + torch.exp(sink.double() - top))[:, None]
+        wants.append((prob @ keys).float())
+        if i == len(q_pos) - 1:
+            assert float(prob[0, far]) > 0.5
+        if p == 0:  # a sequence's first token: its own key and the sink share the weight
+            torch.testing.assert_close(prob[:, 0].float(), torch.sigmoid(score[:, 0].float() - sink))
+    tol = dict(atol=2e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=3e-2, rtol=3e-2)
+    hows = [dict(decode=False)]
+    if dtype == torch.bfloat16 and ops.latent_attention_fits_mfma(R, 0) and (H * R) % 8 == 0:
+        hows += [dict(decode=False, vt_cache=transposed), dict(decode=True, max_context=256, vt_cache=transposed),
+                 dict(decode=True, max_context=8192, vt_cache=transposed)]
+    for how in hows:
+        got = ops.latent_attention(qa.view(len(q_pos), H * R).to(DEV), pos, seq, table, cache, sink.to(DEV), H, R, 0, scale, 0, **how)
+        torch.testing.assert_close(got.float().cpu().view(len(q_pos), H, R), torch.stack(wants), **tol)
+    bare = ops.latent_attention(qa.view(len(q_pos), H * R).to(DEV), pos, seq, table, cache, None, H, R, 0, scale, 0).float().cpu()
+    assert float((bare.view(len(q_pos), H, R) - torch.stack(wants)).abs().max()) > 0.05  # the sink is no no-op here
+
+
+# ---- the engine ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_whole_sequence(lib, folders, name, dtype):
+    from fms_amd.engine import Engine
+
+    ids, want = expected_for(folders, name, 150, 1, dtype)
+    model = get(lib, folders, name, dtype)
+    engine = Engine(model, max_tokens=256, max_slots=2)
+    slot = engine.new_sequence()
+    judge(engine.step([slot], [ids], "all"), want, dtype)
+    engine.end_sequence(slot)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_the_stream_after_every_layer(lib, folders, name):
+    """float32: the residual stream after each layer against the plain implementation's, so that a fault names its layer."""
+    from fms_amd.engine import Engine
+    from fms_amd.engine.model import DecoderModel
+
+    cfg, weights = plain(folders, name)
+    ids = tokens_for(cfg["vocab"], 70, 2)
+    layers = []
+    S.forward(cfg, weights, ids, layers_out=layers)
+    model = get(lib, folders, name, "float32")
+    seen = []
+    blocks = model.layers
+    originals = [b.forward for b in blocks]
+
+    def watch(i):
+        def forward(stream, batch, cache, act_dtype, next_norm=None):
+            originals[i](stream, batch, cache, act_dtype)
+            # what is still pending joins the stream in a copy: the stream after this layer
+            pending, norm = stream.pending, stream.pending_norm
+            joined = S.norm_in_groups(pending.double().cpu(), norm.w["weight"].double().cpu(), norm.groups, norm.eps)
+            seen.append(stream.resid.double().cpu() + joined)
+        return forward
+
+    try:
+        for i, b in enumerate(blocks):
+            b.forward = watch(i)
+        engine = Engine(model, max_tokens=128, max_slots=1)
+        slot = engine.new_sequence()
+        engine.step([slot], [ids], "last")
+        engine.end_sequence(slot)
+    finally:
+        for b in blocks:
+            del b.forward
+    assert isinstance(model, DecoderModel) and len(seen) == len(cfg["layers"])
+    for i, got in enumerate(seen):
+        torch.testing.assert_close(got, layers[i], atol=2e-4, rtol=1e-4, msg=lambda m, i=i: f"layer {i}: {m}")
+
+
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_prompt_then_token_by_token_and_the_first_tokens(lib, folders, name, dtype):
+    from fms_amd.engine import Engine
+
+    ids, want = expected_for(folders, name, 150, 1, dtype)
+    model = get(lib, folders, name, dtype)
+    engine = Engine(model, max_tokens=256, max_slots=2)
+    slot = engine.new_sequence()
+    got = [engine.step([slot], [ids[:100]], "all")] + [engine.step([slot], [[t]], "last") for t in ids[100:]]
+    judge(torch.cat(got), want, dtype)
+    engine.end_sequence(slot)
+    # from the very first token one by one: the first positions of a sequence, where the sink weighs most, the
+    # convolutions still see zeros and the recurrence starts
+    slot = engine.new_sequence()
+    got = [engine.step([slot], [[t]], "last") for t in ids[:40]]
+    judge(torch.cat(got), want[:40], dtype)
+    engine.end_sequence(slot)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_portions_of_several_sizes(lib, folders, name, dtype):
+    from fms_amd.engine import Engine
+
+    ids, want = expected_for(folders, name, 150, 1, dtype)
+    model = get(lib, folders, name, dtype)
+    engine = Engine(model, max_tokens=256, max_slots=1)
+    for cuts in ([2, 2, 60, 1, 63, 2, 20], [64, 64, 22], [63, 2, 2, 83], [1, 127, 22], [3, 1, 1, 2, 143]):
+        slot = engine.new_sequence()
+        got, at = [], 0
+        for n in cuts:
+            got.append(engine.step([slot], [ids[at : at + n]], "all"))
+            at += n
+        assert at == 150
+        judge(torch.cat(got), want, dtype)
+        engine.end_sequence(slot)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_ragged_batches_with_pages_and_slots_used_again(lib, folders, name, dtype):
+    """Unequal requests in one batch, decoded together; the short ones end early, their slots (with the recurrent state
+    and the convolutions' last inputs in them) and pages go to new requests that start while the long one goes on;
+    every request equals itself alone."""
+    from fms_amd.engine import Engine
+
+    lens = {"a": (150, 1), "b": (70, 5), "c": (3, 6), "d": (129, 7), "e": (66, 8)}
+    reqs = {k: expected_for(folders, name, n, seed, dtype) for k, (n, seed) in lens.items()}
+    model = get(lib, folders, name, dtype)
+    engine = Engine(model, max_tokens=64 * 6, max_slots=3)
+    got = {k: [] for k in reqs}
+    slots = {k: engine.new_sequence() for k in ("a", "b", "c")}
+    prompt = {"a": 100, "b": 64, "c": 1}
+    out = engine.step([slots[k] for k in ("a", "b", "c")], [reqs[k][0][: prompt[k]] for k in ("a", "b", "c")], "all")
+    at = 0
+    for k in ("a", "b", "c"):
+        got[k].append(out[at : at + prompt[k]])
+        at += prompt[k]
+    done = dict(prompt)
+    alive = ["a", "b", "c"]
+    waiting = ["d", "e"]
+    while alive:
+        out = engine.step([slots[k] for k in alive], [[reqs[k][0][done[k]]] for k in alive], "last")
+        for i, k in enumerate(alive):
+            got[k].append(out[i : i + 1])
+            done[k] += 1
+        for k in [k for k in alive if done[k] == len(reqs[k][0])]:
+            engine.end_sequence(slots.pop(k))
+            alive.remove(k)
+        if waiting and len(alive) < 2 and "a" in alive:
+            # a batch of its own for the newcomer (the freed slot and pages), then it goes on beside the others
+            k = waiting.pop(0)
+            slots[k] = engine.new_sequence()
+            n = len(reqs[k][0]) - 4
+            got[k].append(engine.step([slots[k]], [reqs[k][0][:n]], "all"))
+            done[k] = n
+            alive.append(k)
+    assert not waiting
+    for k, (ids, want) in reqs.items():
+        judge(torch.cat(got[k]), want, dtype)
+    engine.cache.check()
+    assert engine.cache.n_free_slots == 3 and all(g.pool.n_held == 0 for g in engine.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_far_key_decides_in_prompts_and_in_decoding(lib, dtype, tmp_path):
+    """Queries scaled up: single keys hold most of a query's weight, many of them hundreds of tokens back and on
+    either side of page borders.  A key lost from the cache must fail the same comparison."""
+    from fms_amd.engine import Engine
+
+    cfg_kw = dict(CONFIGS["A"], layers=CONFIGS["A"]["layers"][1:])  # attention first: its scores are formed here from the weights
+    folder = write_folder(lib, str(tmp_path / "sharp"), cfg_kw, seed=21, sharp=160.0)
+    cfg, weights = S.load_model_folder(folder)
+    ids = tokens_for(cfg["vocab"], 600, 3)
+    want = expect(cfg, weights, ids, dtype)
+    model = lib.get_model("hf_pretrained", model_path=folder, data_type=dtype)
+    engine = Engine(model, max_tokens=640, max_slots=1)
+    slot = engine.new_sequence()
+    got = [engine.step([slot], [ids[:520]], "all")] + [engine.step([slot], [[t]], "last") for t in ids[520:]]
+    judge(torch.cat(got), want, dtype)
+    engine.end_sequence(slot)
+    # sharp indeed, and far: layer 0's heaviest key of the late queries
+    m = cfg["layers"][0]["mixer"]
+    w = S.under(weights, "l0.mix.")
+    x = weights["embed"][torch.tensor(ids)]
+    h = x + S.convolution_over_time(x, weights["l0.canon1"])
+    T, H, D = len(ids), m["heads"], m["dim"]
+    q = (h @ w["q"].T).view(T, H, D)
+    latent = S.root_mean_square_norm(h @ w["dkv"].T, cfg["norm"]["eps"]) * w["dkv.norm"]
+    k = (latent @ w["uk"].T).view(T, H, D)
+    pos = torch.arange(T)
+    score = torch.einsum("thd,shd->hts", q, k) * m["scale"]
+    score = score.masked_fill(pos[None, :] > pos[:, None], float("-inf"))
+    prob = torch.softmax(score[:, 520:], -1)
+    heavy = prob.max(-1)
+    decided = heavy.values > 0.5  # (head, late query) pairs whose weight sits on one key
+    assert float(decided.float().mean()) > 0.05 and int((pos[520:][None] - heavy.indices)[decided].max()) > 300
+    # negative control: the key that most late queries lean on is taken out of the cache
+    lost_key = int(torch.mode(heavy.indices[decided]).values)
+    assert lost_key < 520
+    slot = engine.new_sequence()
+    engine.step([slot], [ids[:520]], "last")
+    gi, _ = engine.cache.group_of_entry[0]
+    group = engine.cache.groups[gi]
+    group.keys[:, group.pages[slot][lost_key // 64], :, lost_key % 64, :] = 0
+    lost = torch.cat([engine.step([slot], [[t]], "last") for t in ids[520:]])
+    engine.end_sequence(slot)
+    with pytest.raises(AssertionError):
+        judge(lost, want[520:], dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_state_that_is_lost_shows(lib, folders, dtype):
+    """Negative controls for what a slot carries: the recurrent state set to zero after the prompt, and the stream's
+    last rows that the input convolution reads, each change the decoded logits beyond what the comparison allows."""
+    from fms_amd.engine import Engine
+
+    name = "A"
+    ids, want = expected_for(folders, name, 150, 1, dtype)
+    model = get(lib, folders, name, dtype)
+    engine = Engine(model, max_tokens=256, max_slots=2)
+    # the state of the first recurrent block, its convolution's inputs and the stream's rows in front of it; the same of
+    # a later layer (an attention layer's stream rows matter little where scores are flat: the last layer's are taken)
+    for entry, tensor in ((0, "S"), (0, "conv"), (0, "block.conv"), (3, "S"), (3, "conv"), (4, "block.conv")):
+        slot = engine.new_sequence()
+        engine.step([slot], [ids[:140]], "last")
+        engine.cache.state_of_entry(entry)[tensor][slot].zero_()
+        lost = engine.step([slot], [[ids[140]]], "last")
+        engine.end_sequence(slot)
+        with pytest.raises(AssertionError):
+            judge(lost, want[140:141], dtype)
+    slot = engine.new_sequence()  # the control's control: nothing lost, nothing found
+    engine.step([slot], [ids[:140]], "last")
+    judge(engine.step([slot], [[ids[140]]], "last"), want[140:141], dtype)
+    engine.end_sequence(slot)
+    # the recurrence remembers: the slow channels of layer 0 still hold a good part of what the first tokens brought
+    w = S.under(plain(folders, name)[1], "l0.mix.")
+    slowest = float(torch.exp(-8.0 * torch.nn.functional.softplus(w["lam"])).max())
+    assert slowest ** 100 > 0.3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding_through_graphs_and_eager_steps(lib, folders, dtype):
+    """300 tokens decoded one by one for three sequences of different lengths, across page borders, as captured graphs
+    (fed the plain implementation's tokens through the loop's hook) and as eager steps: the same logits."""
+    from fms_amd.engine import Engine
+    from fms_amd.sampling import SamplingParams
+
+    name = "C"
+    cfg, weights = plain(folders, name)
+    model = get(lib, folders, name, dtype)
+    seqs = [tokens_for(cfg["vocab"], n, 30 + n) for n in (360, 330, 301)]
+    want = [expect(cfg, weights, s, dtype) for s in seqs]
+    for use_graphs in (True, False):
+        engine = Engine(model, max_tokens=64 * 18, max_slots=3, use_graphs=use_graphs)
+        slots = [engine.new_sequence() for _ in seqs]
+        engine.step(slots, [s[: len(s) - 300] for s in seqs], "last")
+        got = [[] for _ in seqs]
+        for i in range(300):
+            feed = [s[len(s) - 300 + i] for s in seqs]
+            if use_graphs:
+                engine.decode_and_choose(slots, feed, SamplingParams(do_sample=False))
+                logits = engine.last_graph.logits[: len(seqs)].clone()
+            else:
+                logits = engine.step(slots, [[t] for t in feed], "last")
+            for b in range(len(seqs)):
+                got[b].append(logits[b : b + 1])
+        for b, s in enumerate(seqs):
+            judge(torch.cat(got[b]), want[b][len(s) - 300 :], dtype)
+        for s in slots:
+            engine.end_sequence(s)
+        engine.cache.check()
+        assert bool(engine.graph_captures) == use_graphs
+
+
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_greedy_generation_through_the_entry_point_and_the_scheduler(lib, folders, name):
+    from fms_amd.engine import Engine
+    from fms_amd.generation import generate, generate_requests
+
+    cfg, weights = plain(folders, name)
+    model = get(lib, folders, name, "float32")
+    prompts = [tokens_for(cfg["vocab"], n, 40 + n) for n in (5, 70, 17, 1)]
+    want = [S.greedy_generate(cfg, weights, p, 12) for p in prompts]
+    for p, w in zip(prompts[:2], want):
+        assert generate(model, torch.tensor(p), max_new_tokens=12, do_sample=False).tolist() == p + w
+    # the scheduler: more requests than slots, so batches follow one another and slots are used again
+    engine = Engine(model, max_tokens=64 * 4, max_slots=2)
+    assert generate_requests(engine, prompts, max_new_tokens=12) == want
+    stop = want[1][5]
+    out = generate_requests(engine, prompts, max_new_tokens=12, stop_token_ids=[stop])
+    for o, w in zip(out, want):
+        assert o == (w[: w.index(stop) + 1] if stop in w else w)
+    engine.cache.check()
+
+
+def test_command_line_and_trace_replay(lib, folders, tmp_path):
+    """The package's programs on a Sidalorn folder: the trace replay (float32 and bfloat16, a batch whose requests end
+    at different steps) and the registry's view of the architecture."""
+    name = "A"
+    cfg, weights = plain(folders, name)
+    assert "sidalorn" in lib.list_models() and "micro" in lib.list_variants("sidalorn")
+    reqs = {"x": tokens_for(cfg["vocab"], 90, 51), "y": tokens_for(cfg["vocab"], 40, 52)}
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": reqs["x"][:80], "want": [0, 79]}, {"id": "y", "tokens": reqs["y"][:38], "want": [37]}], "end": []}]
+    for i in range(10):
+        entries = [{"id": "x", "tokens": [reqs["x"][80 + i]], "want": [0]}]
+        if i < 2:
+            entries.append({"id": "y", "tokens": [reqs["y"][38 + i]], "want": [0] if i == 1 else []})
+        steps.append({"step": i + 1, "entries": entries, "end": (["y"] if i == 1 else []) + (["x"] if i == 9 else [])})
+    for dtype in DTYPES:
+        want = {k: expect(cfg, weights, v, dtype) for k, v in reqs.items()}
+        out_dir = str(tmp_path / f"out_{dtype}")
+        proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folders[name], "--dtype", dtype,
+                               "--out", out_dir, "--max-tokens", "192"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                              capture_output=True, text=True, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert [line for line in proc.stdout.splitlines() if line.startswith("done ")] == [f"done {i}" for i in range(11)]
+
+        def read(step):
+            return torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{step}.f32"), dtype="<f4").reshape(-1, cfg["vocab"]).copy())
+
+        judge(read(0), Expected.stack([want["x"][0], want["x"][79], want["y"][37]]), dtype)
+        judge(read(2), Expected.stack([want["x"][81], want["y"][39]]), dtype)
+        judge(read(10), want["x"][89:90], dtype)
+
+
+def test_the_inference_program_on_a_sidalorn_folder(lib, folders):
+    """bin/fms_inference with a Sidalorn folder and with a registered variant: the model class comes from config.json or
+    from the registry, the text printed is the plain implementation's greedy continuation."""
+    from fms_amd.tokenizers import CharTokenizer
+
+    name = "A"  # its vocabulary holds the character tokenizer's
+    cfg, weights = plain(folders, name)
+    tok = CharTokenizer()
+    prompt = [ord(c) for c in "a gated recurrence"]
+    new = S.greedy_generate(cfg, weights, prompt, 12)
+    if tok.eos_token_id in new:
+        new = new[: new.index(tok.eos_token_id)]
+    env = dict(os.environ, PYTHONIOENCODING="utf-8")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "fms_inference"), "--architecture", "hf_pretrained", "--model_path", folders[name],
+           "--tokenizer", "char_tokenizer", "--default_dtype", "fp32", "--max_new_tokens", "12", "--prompt_ids", ",".join(map(str, prompt))]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=110, env=env)
+    assert proc.returncode == 0, proc.stderr.decode(errors="replace")
+    assert tok.decode(prompt + new) in proc.stdout.decode("utf-8")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "fms_inference"), "--architecture", "sidalorn", "--variant", "micro", "--tokenizer",
+           "char_tokenizer", "--default_dtype", "bf16", "--max_new_tokens", "5", "--prompt_ids", "1,2,3", "--prompt_ids", "7,8"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=110, env=env)
+    assert proc.returncode == 0, proc.stderr.decode(errors="replace")
+    assert "loading complete" in proc.stdout.decode("utf-8")
+
+
+def test_a_model_from_the_registry_alone(lib):
+    """A registered variant with random weights runs: configuration -> parts -> engine, no folder."""
+    from fms_amd.engine import Engine
+
+    model = lib.get_model("sidalorn", "micro", data_type="bfloat16")
+    engine = Engine(model, max_tokens=256, max_slots=2)
+    a, b = engine.new_sequence(), engine.new_sequence()
+    logits = engine.step([a, b], [list(range(70)), [5, 6, 7]], "last")
+    assert logits.shape == (2, model.spec.vocab) and bool(torch.isfinite(logits).all())
+    alone = Engine(model, max_tokens=256, max_slots=1)
+    s = alone.new_sequence()
+    torch.testing.assert_close(alone.step([s], [[5, 6, 7]], "last"), logits[1:], atol=2e-2, rtol=2e-2)
