@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define FMSAMD_ABI_VERSION 5
+#define FMSAMD_ABI_VERSION 6
 
 // element types
 #define FMS_F32 0
@@ -316,6 +316,12 @@ int fmsamd_rglru_gates(const float* u, long ldu, const void* ra_t, const float* 
 int fmsamd_rglru_scan(const float* a, const float* b, const float* y, long ldy, int act, float* state, const int* seq_starts,
                       const int* seq_of_token, const int* slot_ids, void* out, int out_dtype, long ldo, int n_seqs, int channels,
                       hipStream_t stream);
+// Long sequences: the same walk in chunks of token rows that run side by side.  fmsamd_rglru_scan_chunk says how many rows a
+// chunk has for a step (0: walk sequence by sequence); workspace: float32 [(2 * ceil(n_tokens / chunk) + n_seqs) * channels].
+int fmsamd_rglru_scan_chunk(int n_tokens, int n_seqs);
+int fmsamd_rglru_scan_chunked(const float* a, const float* b, const float* y, long ldy, int act, float* state, const int* seq_starts,
+                              const int* seq_of_token, const int* slot_ids, void* out, int out_dtype, long ldo, int n_tokens,
+                              int n_seqs, int channels, int chunk, float* workspace, hipStream_t stream);
 
 #ifdef __cplusplus
 }

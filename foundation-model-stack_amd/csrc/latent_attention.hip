@@ -607,7 +607,7 @@ __global__ void __launch_bounds__(256)
       if (base + 32 <= last_pos) fetch(base + 32);
       // (a condition that all lanes of the wave share: matrix instructions take their operands from every lane)
       if (tile < n_tiles && seq >= 0 && base <= pos) {
-        latent_tile<RT, WC, (WC <= 10 ? WC : 6), (RT <= 16 ? RT : 8), EXACT>(
+        latent_tile<RT, WC, (WC <= 10 ? WC : (WC % 8 == 0 ? 8 : 6)), (RT <= 16 ? RT : 8), EXACT>(
             st, load_q,
             [&](int which, int c) {
               return (EXACT || c * 32 + grp * 8 < width) ? *reinterpret_cast<const bf16x8*>(k_lds + (key_a + 4 * which) * ks + c * 32 + grp * 8) : zero8;
@@ -632,7 +632,7 @@ __global__ void __launch_bounds__(256)
       const bf16* ka = cache + (page * PAGE_TOKENS + in_page + key_a) * width + grp * 8;
       const bf16* vt = vt_cache + (page * rank + col) * PAGE_TOKENS + in_page + grp * 8;
       // straight from global memory: half a tile of key loads, then half its latent loads, in flight at once (all of them up to medium sizes)
-      latent_tile<RT, WC, (WC <= 10 ? WC : 9), (RT <= 16 ? RT : 16), EXACT>(
+      latent_tile<RT, WC, (WC <= 10 ? WC : (WC % 8 == 0 ? 8 : 9)), (RT <= 16 ? RT : 16), EXACT>(
           st, load_q,
           [&](int which, int c) {
             return (EXACT || c * 32 + grp * 8 < width) ? *reinterpret_cast<const bf16x8*>(ka + which * 4 * (size_t)width + c * 32) : zero8;
@@ -737,10 +737,17 @@ extern "C" int fmsamd_latent_attn_mfma(const void* qa, long ldq, void* out, long
     latent_attn_mfma_kernel<RT, WC, false, EXACT><<<grid, 256, q_lds, stream>>>(                                                   \
         (const bf16*)qa, ldq, (bf16*)out, ldo, (float*)workspace, positions, seq_of_token, block_table, table_stride,              \
         (const bf16*)cache, (const bf16*)vt_cache, sink, n_tokens, nheads, rank, width, scale, window, tiles_per_token, n_parts)
-  // the sizes of the largest configuration exactly (a latent of 512 with a rotated part of 64) run without a question
-  // around any product; everything else in the smallest configuration that holds it
+  // the sizes of the largest configuration exactly (a latent of 512 with a rotated part of 64, or with none) and the
+  // smaller latents without a rotated part run without a question around any product; everything else in the smallest
+  // configuration that holds it
   if (rank == 512 && width == 576) {
     LAUNCH_LATENT(32, 18, true);
+  } else if (rank == 512 && width == 512) {
+    LAUNCH_LATENT(32, 16, true);
+  } else if (rank == 256 && width == 256) {
+    LAUNCH_LATENT(16, 8, true);
+  } else if (rank == 128 && width == 128) {
+    LAUNCH_LATENT(8, 4, true);
   } else if (rank <= 128 && width <= 192) {
     LAUNCH_LATENT(8, 6, false);
   } else if (rank <= 256 && width <= 320) {

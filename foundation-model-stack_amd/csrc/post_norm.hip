@@ -131,6 +131,91 @@ __global__ void __launch_bounds__(1024)
   }
 }
 
+// Steps of many tokens: a block takes CONV_TILE consecutive token rows and a thread VEC neighbouring channels, whose last
+// inputs it carries from row to row in registers, so every input is loaded once.  A sequence's start inside the tile (and
+// the tile's first row) fills the registers from the rows before, or from the state where the step holds no more.  The
+// convolution is run as one of CONV_MAX_TAPS taps whose first weights are zero: every register has a fixed place.
+#define CONV_TILE 16
+
+template <typename W, typename T, int VEC>
+__global__ void __launch_bounds__(256)
+    short_conv_tile_kernel(const float* __restrict__ x, long ld, int C, const W* __restrict__ conv_w, const W* __restrict__ bias,
+                           int taps, const float* __restrict__ conv_state, const int* __restrict__ seq_of_token,
+                           const int* __restrict__ slot_ids, int add_input, T* __restrict__ out, long ldo, int n_tokens) {
+  const int c0 = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
+  if (c0 >= C) return;
+  const int first = blockIdx.x * CONV_TILE, last = min(first + CONV_TILE, n_tokens);
+  // back[d][v]: the weight of the input d rows back (d = 0: the row's own), hist[d - 1][v]: that input
+  float back[CONV_MAX_TAPS][VEC], hist[CONV_MAX_TAPS - 1][VEC], bv[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    bv[v] = bias ? to_f32(bias[c0 + v]) : 0.f;
+#pragma unroll
+    for (int d = 0; d < CONV_MAX_TAPS; ++d) back[d][v] = d < taps ? to_f32(conv_w[(size_t)(c0 + v) * taps + (taps - 1 - d)]) : 0.f;
+#pragma unroll
+    for (int d = 0; d < CONV_MAX_TAPS - 1; ++d) hist[d][v] = 0.f;
+  }
+  float xs[CONV_TILE][VEC];  // the tile's rows, asked for together
+#pragma unroll
+  for (int e = 0; e < CONV_TILE; ++e) {
+    const int t = first + e;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) xs[e][v] = 0.f;
+    if (t < last) {
+      if (VEC == 4) {
+        const float4 q = *reinterpret_cast<const float4*>(x + (size_t)t * ld + c0);
+        xs[e][0] = q.x, xs[e][1] = q.y, xs[e][2] = q.z, xs[e][3] = q.w;
+      } else {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) xs[e][v] = x[(size_t)t * ld + c0 + v];
+      }
+    }
+  }
+  int prev = -2;
+#pragma unroll
+  for (int e = 0; e < CONV_TILE; ++e) {
+    const int t = first + e;
+    if (t >= last) break;
+    const int seq = seq_of_token[t];
+    T* o = out + (size_t)t * ldo + c0;
+    if (seq < 0) {  // a padding row
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) o[v] = from_f32<T>(0.f);
+      prev = seq;
+      continue;
+    }
+    if (seq != prev) {  // the tile's first row, or a sequence's first row of the step
+      const int have = tokens_before(seq_of_token, t, seq, taps);
+      const float* state = conv_state + (size_t)slot_ids[seq] * (taps - 1) * C;
+#pragma unroll
+      for (int d = 1; d < CONV_MAX_TAPS; ++d) {
+        if (d < taps) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v)
+            hist[d - 1][v] = d <= have ? x[(size_t)(t - d) * ld + c0 + v] : state[(size_t)(taps - 1 + have - d) * C + c0 + v];
+        }
+      }
+    }
+    prev = seq;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      float acc = bv[v];
+#pragma unroll
+      for (int d = CONV_MAX_TAPS - 1; d > 0; --d) acc = fmaf(back[d][v], hist[d - 1][v], acc);  // the oldest input first
+      acc = fmaf(back[0][v], xs[e][v], acc);
+      if (add_input) acc += xs[e][v];
+      o[v] = from_f32<T>(acc);  // the same sums in the same order as the kernel of short steps
+    }
+#pragma unroll
+    for (int d = CONV_MAX_TAPS - 2; d > 0; --d) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) hist[d][v] = hist[d - 1][v];
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) hist[0][v] = xs[e][v];
+  }
+}
+
 extern "C" int fmsamd_short_conv(const float* x, long ld, int channels, const void* conv_w, const void* bias, int weight_dtype,
                                  int taps, float* conv_state, const int* seq_of_token, const int* slot_ids, int add_input,
                                  void* out, int out_dtype, long ldo, int n_tokens, hipStream_t stream) {
@@ -140,6 +225,33 @@ extern "C" int fmsamd_short_conv(const float* x, long ld, int channels, const vo
   FMS_REQUIRE(taps >= 1 && taps <= CONV_MAX_TAPS, "short_conv: %d taps (1 to %d)", taps, CONV_MAX_TAPS);
   FMS_REQUIRE(taps == 1 || conv_state != nullptr, "short_conv: a convolution of %d taps needs the sequences' state", taps);
   const int threads = n_tokens <= 64 ? 1024 : 256;
+  if (n_tokens >= 4 * CONV_TILE) {  // many rows: tiles of rows, every input loaded once
+    const bool wide = channels % 4 == 0 && ld % 4 == 0 && ((uintptr_t)x % 16) == 0;
+    const int per_block = 256 * (wide ? 4 : 1);
+    const dim3 grid(ceil_div(n_tokens, CONV_TILE), ceil_div(channels, per_block));
+    FMS_REQUIRE(grid.y <= 65535, "short_conv: %d channels are too many for one launch", channels);
+#define FMS_CONV_TILE(W, T)                                                                                                          \
+  do {                                                                                                                               \
+    if (wide)                                                                                                                        \
+      short_conv_tile_kernel<W, T, 4><<<grid, 256, 0, stream>>>(x, ld, channels, (const W*)conv_w, (const W*)bias, taps, conv_state, \
+                                                                seq_of_token, slot_ids, add_input, (T*)out, ldo, n_tokens);          \
+    else                                                                                                                             \
+      short_conv_tile_kernel<W, T, 1><<<grid, 256, 0, stream>>>(x, ld, channels, (const W*)conv_w, (const W*)bias, taps, conv_state, \
+                                                                seq_of_token, slot_ids, add_input, (T*)out, ldo, n_tokens);          \
+  } while (0)
+    if (weight_dtype == FMS_F32 && out_dtype == FMS_F32) FMS_CONV_TILE(float, float);
+    else if (weight_dtype == FMS_F32 && out_dtype == FMS_BF16) FMS_CONV_TILE(float, bf16);
+    else if (weight_dtype == FMS_BF16 && out_dtype == FMS_F32) FMS_CONV_TILE(bf16, float);
+    else if (weight_dtype == FMS_BF16 && out_dtype == FMS_BF16) FMS_CONV_TILE(bf16, bf16);
+    else FMS_REQUIRE(false, "short_conv: unknown dtypes %d %d", weight_dtype, out_dtype);
+#undef FMS_CONV_TILE
+    FMS_LAUNCH_CHECK("short_conv_tile");
+    if (taps > 1) {
+      conv_state_kernel<<<n_tokens, threads, 0, stream>>>(x, ld, taps, conv_state, seq_of_token, slot_ids, n_tokens, channels);
+      FMS_LAUNCH_CHECK("conv_state");
+    }
+    return 0;
+  }
 #define FMS_CONV(W, T)                                                                                                     \
   short_conv_kernel<W, T><<<n_tokens, threads, 0, stream>>>(x, ld, channels, (const W*)conv_w, (const W*)bias, taps, conv_state, \
                                                             seq_of_token, slot_ids, add_input, (T*)out, ldo)

@@ -17,7 +17,7 @@ import torch  # noqa: F401  (loads libamdhip64 before our library asks for it)
 
 from . import build as _build
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
@@ -65,6 +65,8 @@ _SIGNATURES = {
     "fmsamd_short_conv": [P, L, I, P, P, I, I, P, P, P, I, P, I, L, I, P],
     "fmsamd_rglru_gates": [P, L, P, P, P, P, I, P, F, P, P, P, I, I, I, P],
     "fmsamd_rglru_scan": [P, P, P, L, I, P, P, P, P, P, I, L, I, I, P],
+    "fmsamd_rglru_scan_chunk": [I, I],
+    "fmsamd_rglru_scan_chunked": [P, P, P, L, I, P, P, P, P, P, I, L, I, I, I, I, P, P],
     "fmsamd_qk_projection_norm": [P, L, I, I, I, P, P, I, F, P, I, L, P, I, P],
     "fmsamd_gate_mul": [P, L, P, L, I, F, P, L, I, I, I, P],
     "fmsamd_scale_f32": [P, L, F, P],

@@ -788,8 +788,17 @@ def rglru_scan(a: torch.Tensor, b: torch.Tensor, y: torch.Tensor, activation: st
         raise ValueError(f"the state is contiguous float32 [slots, {C}]")
     if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs or seq_of_token.numel() < T:
         raise ValueError("the step's index arrays are shorter than its sequences or tokens")
+    lib = load()
+    chunk = lib.fmsamd_rglru_scan_chunk(T, int(n_seqs))
+    if chunk:  # long sequences: chunks of token rows side by side (they cover every row, padding rows come back as zeros)
+        out = torch.empty(T, C, dtype=out_dtype, device=a.device)
+        ws = torch.empty((2 * -(-T // chunk) + int(n_seqs)) * C, dtype=torch.float32, device=a.device)
+        check(lib.fmsamd_rglru_scan_chunked(a.data_ptr(), b.data_ptr(), y.data_ptr(), y.stride(0), ACTIVATIONS[activation], state.data_ptr(),
+                                            seq_starts.data_ptr(), seq_of_token.data_ptr(), slot_ids.data_ptr(), out.data_ptr(),
+                                            _code(out_dtype), out.stride(0), T, int(n_seqs), C, chunk, ws.data_ptr(), _stream()))
+        return out
     out = (torch.zeros if zero_rows else torch.empty)(T, C, dtype=out_dtype, device=a.device)
-    check(load().fmsamd_rglru_scan(a.data_ptr(), b.data_ptr(), y.data_ptr(), y.stride(0), ACTIVATIONS[activation], state.data_ptr(),
+    check(lib.fmsamd_rglru_scan(a.data_ptr(), b.data_ptr(), y.data_ptr(), y.stride(0), ACTIVATIONS[activation], state.data_ptr(),
                                    seq_starts.data_ptr(), seq_of_token.data_ptr(), slot_ids.data_ptr(), out.data_ptr(), _code(out_dtype),
                                    out.stride(0), int(n_seqs), C, _stream()))
     return out

@@ -304,7 +304,9 @@ def test_convolution_over_time_in_steps_of_any_cut(lib, out_dtype, sizes):
 
 
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(12, 3, 5), (60, 5, 19), (128, 1, 8), (384, 3, 33), (64, 64, 7), (1024, 2, 3)])
+# the last three: steps of many tokens and blocks too wide for the kernel of small steps (the tiled kernel runs)
+@pytest.mark.parametrize("sizes", [(12, 3, 5), (60, 5, 19), (128, 1, 8), (384, 3, 33), (64, 64, 7), (1024, 2, 3), (64, 2, 4100), (2048, 1, 9),
+                                   (120, 3, 3000)])
 def test_gates_of_the_recurrence(lib, wdtype, sizes):
     from fms_amd.kernels import ops
 
@@ -373,6 +375,49 @@ def test_recurrence_in_steps_of_any_cut(lib, out_dtype, C):
     final = S.linear_recurrence(a[0].double(), b[0].double())[-1].float()
     torch.testing.assert_close(state[3].cpu(), final, atol=2e-5, rtol=2e-5)
     assert float(final[0]) > 100.0 and float((state[1] - 3.0).abs().max()) == 0.0  # the first token is still there; other slots untouched
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [(12, (700, 130, 400)), (300, (256,)), (64, (9000, 1000)), (1024, (64, 1, 63, 2, 1500)), (5, (40000,))])
+def test_recurrence_over_long_steps_in_chunks(lib, out_dtype, sizes):
+    """Steps long enough to be walked in chunks of rows side by side: several sequences in one step with their borders
+    inside chunks and at chunk borders, each from a state that an earlier step left, one decay close to one."""
+    from fms_amd.kernels import ops
+
+    C, lens = sizes
+    gen = torch.Generator().manual_seed(C + len(lens))
+    before = 3  # tokens of every sequence in a first, short step
+    a = [torch.rand(n + before, C, generator=gen) for n in lens]
+    b = [torch.randn(n + before, C, generator=gen) for n in lens]
+    y = [torch.randn(n + before, C + 4, generator=gen) for n in lens]
+    # a slow channel that carries a large first input across all chunks (over tens of thousands of tokens a decay this
+    # close to one lets float32 rounding add up beyond the tolerance below, in any order of evaluation: slower there)
+    a[0][:, 0] = 0.9999 if sum(lens) < 5000 else 0.999
+    b[0][0, 0] = 300.0 if sum(lens) < 5000 else 20.0
+    want = [S.linear_recurrence(a[s].double(), b[s].double()).float() * S.gelu_tanh(y[s][:, 1 : 1 + C].double()).float() for s in range(len(lens))]
+    state = torch.full((len(lens) + 2, C), 3.0, device=DEV)
+    slots = list(range(len(lens), 0, -1))
+    for s in slots:
+        state[s].zero_()
+    got = []
+    for lo, hi in ((0, before), (before, None)):
+        ns = [(hi if hi is not None else len(a[s])) - lo for s in range(len(lens))]
+        starts = [0]
+        for n in ns:
+            starts.append(starts[-1] + n)
+        cat = lambda parts: torch.cat([p[lo : lo + n] for p, n in zip(parts, ns)]).contiguous().to(DEV)  # noqa: E731
+        yy = cat(y)
+        out = ops.rglru_scan(cat(a), cat(b), yy[:, 1 : 1 + C], "gelu-tanh", state, _i32(starts), _i32([j for j, n in enumerate(ns) for _ in range(n)]),
+                             _i32(slots), len(lens), out_dtype)
+        got.append([out[starts[j] : starts[j + 1]].float().cpu() for j in range(len(lens))])
+    assert ops.load().fmsamd_rglru_scan_chunk(sum(lens), len(lens)) > 0  # the second step was walked in chunks
+    # float32: the slow channel sums the rounding of a thousand tokens and more
+    tol = dict(atol=2e-4, rtol=5e-5) if out_dtype == torch.float32 else dict(atol=3e-2, rtol=1e-2)
+    for s in range(len(lens)):
+        torch.testing.assert_close(torch.cat([got[0][s], got[1][s]]), want[s], **tol)
+        final = S.linear_recurrence(a[s].double(), b[s].double())[-1].float()
+        torch.testing.assert_close(state[slots[s]].cpu(), final, atol=2e-4, rtol=5e-5)
+    assert float((state[0] - 3.0).abs().max()) == 0.0 and float((state[-1] - 3.0).abs().max()) == 0.0  # other slots untouched
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
