@@ -303,6 +303,53 @@ def test_convolution_over_time_in_steps_of_any_cut(lib, out_dtype, sizes):
         assert float((state[0] - 9.0).abs().max()) == 0.0  # other slots are not touched
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [(4, 128, True), (3, 101, False), (8, 260, True), (1, 64, True), (2, 1030, False)])
+def test_convolution_over_time_in_long_steps(lib, out_dtype, sizes):
+    """Steps long enough for the kernel that walks tiles of rows: sequences that start at tile borders, just before and
+    just behind them, one of a single token, each after a first step of two tokens whose inputs wait in the state; the
+    same numbers as the kernel of short steps gives token by token."""
+    from fms_amd.kernels import ops
+
+    taps, C, add_input = sizes
+    gen = torch.Generator().manual_seed(taps * 1000 + C)
+    lens = [16 * 3 - 1, 1, 16, 2, 200, 15, 70]  # starts at rows 0, 47, 48, 64, 66, 266, 281 of the long step
+    xs = [torch.randn(n + 2, C + 8, generator=gen) for n in lens]
+    w = torch.randn(C, taps, generator=gen)
+    bias = None if add_input else torch.randn(C, generator=gen)
+    want = [S.convolution_over_time(x[:, 4 : 4 + C].double(), w.double(), None if bias is None else bias.double()).float()
+            + (x[:, 4 : 4 + C] if add_input else 0) for x in xs]
+    slots = [5, 0, 3, 7, 1, 6, 2]
+
+    def run(state, steps):
+        got = [[] for _ in lens]
+        for lo, hi in steps:
+            ns = [min(hi, len(x)) - lo for x in xs]
+            keep = [j for j, n in enumerate(ns) if n > 0]
+            x = torch.cat([xs[j][lo : lo + ns[j]] for j in keep]).to(DEV)
+            out = ops.short_conv(x, 4, C, w.to(DEV), None if bias is None else bias.to(DEV), state, _i32([i for i, j in enumerate(keep) for _ in range(ns[j])]),
+                                 _i32([slots[j] for j in keep]), out_dtype, add_input=add_input)
+            at = 0
+            for j in keep:
+                got[j].append(out[at : at + ns[j]].float().cpu())
+                at += ns[j]
+        return [torch.cat(g) for g in got]
+
+    new_state = lambda: torch.zeros(8, max(taps - 1, 1), C, device=DEV) if taps > 1 else None  # noqa: E731
+    state = new_state()
+    long_steps = run(state, [(0, 2), (2, 1000)])
+    tol = dict(atol=1e-5, rtol=1e-5) if out_dtype == torch.float32 else dict(atol=3e-2, rtol=1e-2)
+    for j in range(len(lens)):
+        torch.testing.assert_close(long_steps[j], want[j], **tol)
+    one_by_one_state = new_state()
+    one_by_one = run(one_by_one_state, [(t, t + 1) for t in range(202)])
+    for j in range(len(lens)):
+        assert torch.equal(long_steps[j], one_by_one[j])
+    if taps > 1:
+        assert torch.equal(state, one_by_one_state)
+        torch.testing.assert_close(state[1].cpu(), xs[4][-(taps - 1):, 4 : 4 + C])
+
+
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
 # the last three: steps of many tokens and blocks too wide for the kernel of small steps (the tiled kernel runs)
 @pytest.mark.parametrize("sizes", [(12, 3, 5), (60, 5, 19), (128, 1, 8), (384, 3, 33), (64, 64, 7), (1024, 2, 3), (64, 2, 4100), (2048, 1, 9),
