@@ -207,10 +207,81 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// Rows of at most THREADS * 4 * NV elements (a multiple of 4, rows 16 bytes aligned): a thread keeps its NV groups of four
+// elements in registers, so the row is read once, and the three sums are reduced together.
+template <typename T, int NV>
+__global__ void __launch_bounds__(1024)
+    poly_norm_reg_kernel(const float* __restrict__ z, long ldz, int n, float a, float b, float c, float e, float eps,
+                         T* __restrict__ out, long ldo) {
+  __shared__ float sums[3][16];
+  const float* zr = z + (size_t)blockIdx.x * ldz;
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, nwaves = blockDim.x / WAVE;
+  float4 v[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int i = (k * blockDim.x + threadIdx.x) * 4;
+    v[k] = i < n ? *reinterpret_cast<const float4*>(zr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const float q[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float v2 = q[j] * q[j], v3 = v2 * q[j];
+      s2 = fmaf(q[j], q[j], s2);
+      s4 = fmaf(v2, v2, s4);
+      s6 = fmaf(v3, v3, s6);
+    }
+  }
+  s2 = wave_sum(s2), s4 = wave_sum(s4), s6 = wave_sum(s6);
+  if (lane == 0) sums[0][wave] = s2, sums[1][wave] = s4, sums[2][wave] = s6;
+  __syncthreads();
+  float t2 = 0.f, t4 = 0.f, t6 = 0.f;
+  for (int w = 0; w < nwaves; ++w) t2 += sums[0][w], t4 += sums[1][w], t6 += sums[2][w];  // the same order in every thread
+  const float r1 = a * rsqrtf(t2 / (float)n + eps), r2 = b * rsqrtf(t4 / (float)n + eps), r3 = c * rsqrtf(t6 / (float)n + eps);
+  T* o = out + (size_t)blockIdx.x * ldo;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int i = (k * blockDim.x + threadIdx.x) * 4;
+    if (i < n) {
+      const float q[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+      f32x4 r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float v2 = q[j] * q[j];
+        r[j] = fmaf(r1, q[j], fmaf(r2, v2, fmaf(r3, v2 * q[j], e)));
+      }
+      store4(o + i, r);
+    }
+  }
+}
+
 extern "C" int fmsamd_poly_norm(const float* z, long ldz, int n, float a, float b, float c, float e, float eps, void* out,
                                 int out_dtype, long ldo, int rows, hipStream_t stream) {
   if (rows == 0) return 0;
   FMS_REQUIRE(rows > 0 && n > 0 && ldz >= n && ldo >= n, "poly_norm: bad sizes rows=%d n=%d ldz=%ld ldo=%ld", rows, n, ldz, ldo);
+  // a step of few rows has few blocks: more threads a row
+  const int threads = rows <= 128 ? 1024 : 256;
+  const int nv = ceil_div(n, threads * 4);
+  const size_t esize = out_dtype == FMS_F32 ? 4 : 2;
+  if (n % 4 == 0 && ldz % 4 == 0 && ldo % 4 == 0 && ((uintptr_t)z % 16) == 0 && ((uintptr_t)out % (4 * esize)) == 0 && nv <= 8 &&
+      (out_dtype == FMS_F32 || out_dtype == FMS_BF16)) {
+#define FMS_POLY(NV)                                                                                                       \
+  do {                                                                                                                     \
+    if (out_dtype == FMS_F32)                                                                                              \
+      poly_norm_reg_kernel<float, NV><<<rows, threads, 0, stream>>>(z, ldz, n, a, b, c, e, eps, (float*)out, ldo);         \
+    else                                                                                                                   \
+      poly_norm_reg_kernel<bf16, NV><<<rows, threads, 0, stream>>>(z, ldz, n, a, b, c, e, eps, (bf16*)out, ldo);           \
+  } while (0)
+    if (nv <= 1) FMS_POLY(1);
+    else if (nv <= 2) FMS_POLY(2);
+    else if (nv <= 4) FMS_POLY(4);
+    else FMS_POLY(8);
+#undef FMS_POLY
+    FMS_LAUNCH_CHECK("poly_norm_reg");
+    return 0;
+  }
   if (out_dtype == FMS_F32)
     poly_norm_kernel<float><<<rows, 256, 0, stream>>>(z, ldz, n, a, b, c, e, eps, (float*)out, ldo);
   else if (out_dtype == FMS_BF16)

@@ -69,6 +69,130 @@ __global__ void __launch_bounds__(256)
   for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = from_f32<T>(row[i] * inv[i / part] * scale_at(w, w_dtype, i));
 }
 
+// Four consecutive elements of a row, or of a weight given with its type's code, as floats in one load; and back.
+template <typename T>
+__device__ __forceinline__ f32x4 row4(const T* p) {
+  if constexpr (sizeof(T) == 4) {
+    return *reinterpret_cast<const f32x4*>(p);
+  } else {
+    const bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+    return f32x4{(float)t[0], (float)t[1], (float)t[2], (float)t[3]};
+  }
+}
+__device__ __forceinline__ f32x4 weight4(const void* w, int dtype, int i) {
+  return dtype == FMS_F32 ? row4((const float*)w + i) : row4((const bf16*)w + i);
+}
+template <typename T>
+__device__ __forceinline__ void put4(T* p, f32x4 v) {
+  if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<f32x4*>(p) = v;
+  } else {
+    *reinterpret_cast<bf16x4*>(p) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+  }
+}
+
+// The same for rows of at most 1024 * KEEP elements whose groups are multiples of 256 elements: branch, stream and both
+// weights are asked for at once, four elements a load, and wait in registers, so the kernel pays the memory's latency
+// once (a decode step's rows are few, and nothing else hides it) and reads every row once.  A wave's 256 elements of a
+// pass lie in one group: the waves leave their sums of squares in LDS, and a group's scale is the sum of its waves' in
+// a fixed order.  Rows of a prompt and of a decode step run this same kernel.
+template <typename T, int KEEP>
+__global__ void __launch_bounds__(256)
+    group_norm_chain_small_kernel(float* __restrict__ resid, const T* __restrict__ branch, const void* __restrict__ wb, int wb_dtype,
+                                  int groups_b, float eps_b, const void* __restrict__ w, int w_dtype, int groups, float eps,
+                                  T* __restrict__ out, int out_mode, const int* __restrict__ rows, int width) {
+  __shared__ float partial[4 * KEEP];
+  const int r = rows ? rows[blockIdx.x] : blockIdx.x;
+  float* x = resid + (size_t)r * width;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const f32x4 ones = {1.f, 1.f, 1.f, 1.f}, zeros = {0.f, 0.f, 0.f, 0.f};
+  f32x4 bv[KEEP], xv[KEEP], wbv[KEEP], wv[KEEP];
+#pragma unroll
+  for (int n = 0; n < KEEP; ++n) {
+    const int i = (threadIdx.x + n * 256) * 4;
+    bv[n] = zeros, xv[n] = zeros, wbv[n] = ones, wv[n] = ones;
+    if (i < width) {
+      xv[n] = row4(x + i);
+      if (branch) bv[n] = row4(branch + (size_t)r * width + i);
+      if (branch && groups_b > 0 && wb) wbv[n] = weight4(wb, wb_dtype, i);
+      if (out_mode == FMS_CHAIN_NORM && w) wv[n] = weight4(w, w_dtype, i);
+    }
+  }
+  if (branch != nullptr) {
+    if (groups_b > 0) {
+#pragma unroll
+      for (int n = 0; n < KEEP; ++n) {
+        float sq = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sq = fmaf(bv[n][e], bv[n][e], sq);
+        sq = wave_sum(sq);
+        if (lane == 0) partial[n * 4 + wave] = sq;
+      }
+      __syncthreads();
+      const int part = width / groups_b, per = part / 256;
+#pragma unroll
+      for (int n = 0; n < KEEP; ++n) {
+        const int i = (threadIdx.x + n * 256) * 4;
+        if (i < width) {
+          const int p0 = (i / part) * per;
+          float sum = 0.f;
+          for (int p = p0; p < p0 + per; ++p) sum += partial[p];
+          const float inv = rsqrtf(sum / (float)part + eps_b);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) xv[n][e] = xv[n][e] + bv[n][e] * inv * wbv[n][e];
+        }
+      }
+      __syncthreads();  // the sums are read: the next norm may write its own
+    } else {
+#pragma unroll
+      for (int n = 0; n < KEEP; ++n)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) xv[n][e] += bv[n][e];
+    }
+    if (!rows) {
+#pragma unroll
+      for (int n = 0; n < KEEP; ++n) {
+        const int i = (threadIdx.x + n * 256) * 4;
+        if (i < width) put4(x + i, xv[n]);
+      }
+    }
+  }
+  if (out_mode == FMS_CHAIN_NONE) return;
+  T* o = out + (size_t)blockIdx.x * width;
+  if (out_mode == FMS_CHAIN_CAST) {
+#pragma unroll
+    for (int n = 0; n < KEEP; ++n) {
+      const int i = (threadIdx.x + n * 256) * 4;
+      if (i < width) put4(o + i, xv[n]);
+    }
+    return;
+  }
+#pragma unroll
+  for (int n = 0; n < KEEP; ++n) {
+    float sq = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sq = fmaf(xv[n][e], xv[n][e], sq);
+    sq = wave_sum(sq);
+    if (lane == 0) partial[n * 4 + wave] = sq;
+  }
+  __syncthreads();
+  const int part = width / groups, per = part / 256;
+#pragma unroll
+  for (int n = 0; n < KEEP; ++n) {
+    const int i = (threadIdx.x + n * 256) * 4;
+    if (i < width) {
+      const int p0 = (i / part) * per;
+      float sum = 0.f;
+      for (int p = p0; p < p0 + per; ++p) sum += partial[p];
+      const float inv = rsqrtf(sum / (float)part + eps);
+      f32x4 y;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[e] = xv[n][e] * inv * wv[n][e];
+      put4(o + i, y);
+    }
+  }
+}
+
 extern "C" int fmsamd_group_norm_chain(float* resid, const void* branch, int act_dtype, const void* branch_weight,
                                        int branch_weight_dtype, int branch_groups, float branch_eps, const void* weight,
                                        int weight_dtype, int groups, float eps, void* out, int out_mode, const int* rows,
@@ -82,6 +206,22 @@ extern "C" int fmsamd_group_norm_chain(float* resid, const void* branch, int act
               "group_norm_chain: %d groups do not divide the branch's %d channels", branch_groups, width);
   FMS_REQUIRE(out_mode != FMS_CHAIN_NORM || (groups > 0 && groups <= 1024 && width % groups == 0),
               "group_norm_chain: %d groups do not divide %d channels", groups, width);
+  const bool branch_fits = branch == nullptr || branch_groups == 0 || (width / branch_groups) % 256 == 0;
+  const bool norm_fits = out_mode != FMS_CHAIN_NORM || (width / groups) % 256 == 0;
+  const bool types_fit = (branch_weight == nullptr || branch_weight_dtype == FMS_F32 || branch_weight_dtype == FMS_BF16) &&
+                         (weight == nullptr || weight_dtype == FMS_F32 || weight_dtype == FMS_BF16);
+  if (width <= 1024 * 4 && width % 4 == 0 && branch_fits && norm_fits && types_fit && (act_dtype == FMS_F32 || act_dtype == FMS_BF16)) {
+    if (act_dtype == FMS_F32)
+      group_norm_chain_small_kernel<float, 4><<<n_out, 256, 0, stream>>>(resid, (const float*)branch, branch_weight, branch_weight_dtype,
+                                                                         branch_groups, branch_eps, weight, weight_dtype, groups, eps,
+                                                                         (float*)out, out_mode, rows, width);
+    else
+      group_norm_chain_small_kernel<bf16, 4><<<n_out, 256, 0, stream>>>(resid, (const bf16*)branch, branch_weight, branch_weight_dtype,
+                                                                        branch_groups, branch_eps, weight, weight_dtype, groups, eps,
+                                                                        (bf16*)out, out_mode, rows, width);
+    FMS_LAUNCH_CHECK("group_norm_chain_small");
+    return 0;
+  }
   const size_t lds = ((size_t)width + 1024) * sizeof(float);
   if (act_dtype == FMS_F32)
     group_norm_chain_kernel<float><<<n_out, 256, lds, stream>>>(resid, (const float*)branch, branch_weight, branch_weight_dtype,

@@ -217,7 +217,10 @@ def _i32(values):
 
 # ---- mechanisms alone ------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(40, 1, 1), (192, 4, 2), (1000, 5, 8), (3000, 3, 1), (4096, 8, 4), (36, 36, 6)])
+# (width, the branch norm's groups, the next norm's groups); the last four: groups of whole multiples of 256 elements in rows
+# of at most 4096, which a kernel of its own keeps in registers
+@pytest.mark.parametrize("sizes", [(40, 1, 1), (192, 4, 2), (1000, 5, 8), (3000, 3, 1), (8192, 8, 4), (36, 36, 6), (4096, 8, 4), (2048, 4, 1),
+                                   (1024, 1, 4), (768, 3, 1)])
 def test_norm_in_groups_behind_a_branch_the_sum_and_what_is_read_next(lib, dtype, sizes):
     from fms_amd.kernels import ops
 
@@ -468,11 +471,14 @@ def test_recurrence_over_long_steps_in_chunks(lib, out_dtype, sizes):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n", [20, 160, 1001, 5000])
-def test_polynorm(lib, out_dtype, n):
+@pytest.mark.parametrize("shape", [(6, 20), (6, 160), (6, 1001), (6, 5000), (6, 8192), (3, 32768), (3, 40000), (140, 320), (140, 8192), (140, 9000)])
+def test_polynorm(lib, out_dtype, shape):
+    """Rows that a thread block keeps in registers (multiples of 4 up to 32768 elements in steps of few rows, up to 8192
+    in steps of many) and rows that it reads twice."""
     from fms_amd.kernels import ops
 
-    z = torch.randn(6, n + 3, generator=torch.Generator().manual_seed(n)) * 2
+    rows, n = shape
+    z = torch.randn(rows, n + (4 if n % 4 == 0 else 3), generator=torch.Generator().manual_seed(n)) * 2
     z[1] *= 30  # rows of very different sizes: every row has its own three root mean squares
     z[2] *= 0.01
     coefficients = (0.7, -0.4, 0.25, 0.1)
