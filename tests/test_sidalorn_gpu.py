@@ -714,7 +714,7 @@ def drawn_configuration(seed):
             blocks = int(pick(1, 2, 4, 5, 8))
             mixer = recurrent(blocks * int(pick(8, 12, 16, 32, 64)), blocks, int(pick(1, 2, 3, 4, 6)))
         layers.append(layer(mixer, feed_forward()))
-    return dict(vocab=int(pick(200, 333, 448, 1000)), width=width, norm={"eps": float(pick(1e-5, 1e-6, 1e-3)), "groups": norm_groups},
+    return dict(vocab=int(pick(200, 333, 480, 1000)), width=width, norm={"eps": float(pick(1e-5, 1e-6, 1e-3)), "groups": norm_groups},
                 canon={"taps": int(pick(1, 2, 3, 4, 6))}, max_positions=1024, layers=layers)
 
 
