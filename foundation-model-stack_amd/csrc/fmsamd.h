@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define FMSAMD_ABI_VERSION 6
+#define FMSAMD_ABI_VERSION 7
 
 // element types
 #define FMS_F32 0
@@ -301,9 +301,10 @@ int fmsamd_group_norm_chain(float* resid, const void* branch, int act_dtype, con
                             void* out, int out_mode, const int* rows, int n_out, int width, hipStream_t stream);
 // out[t, c] = (x[t, c] if add_input) + bias[c] + sum_j conv_w[c, j] x[t - taps + 1 + j, c] over a sequence's own tokens; the
 // inputs before the step come from conv_state [slots][taps-1][channels] (float32), which is then moved on.  x: float32 rows.
+// single_tokens: the caller knows that every sequence brings one token (a short step then needs no second kernel for the state).
 int fmsamd_short_conv(const float* x, long ld, int channels, const void* conv_w, const void* bias, int weight_dtype, int taps,
                       float* conv_state, const int* seq_of_token, const int* slot_ids, int add_input, void* out, int out_dtype,
-                      long ldo, int n_tokens, hipStream_t stream);
+                      long ldo, int n_tokens, int single_tokens, hipStream_t stream);
 
 // ---- the real-gated linear recurrent unit (rglru.hip) -------------------------------------------------------------------
 // u: float32 rows; ra_t, ri_t [blocks][in][out] (transposed square matrices), ra_b, ri_b, lam float32 [channels];

@@ -241,8 +241,8 @@ extern "C" int fmsamd_group_norm_chain(float* resid, const void* branch, int act
 template <typename W, typename T>
 __global__ void __launch_bounds__(1024)
     short_conv_kernel(const float* __restrict__ x, long ld, int C, const W* __restrict__ conv_w, const W* __restrict__ bias,
-                      int taps, const float* __restrict__ conv_state, const int* __restrict__ seq_of_token,
-                      const int* __restrict__ slot_ids, int add_input, T* __restrict__ out, long ldo) {
+                      int taps, float* __restrict__ conv_state, const int* __restrict__ seq_of_token,
+                      const int* __restrict__ slot_ids, int add_input, T* __restrict__ out, long ldo, int move_state) {
   const int t = blockIdx.x;
   const int seq = seq_of_token[t];
   T* o = out + (size_t)t * ldo;
@@ -251,7 +251,7 @@ __global__ void __launch_bounds__(1024)
     return;
   }
   const int have = tokens_before(seq_of_token, t, seq, taps);
-  const float* state = conv_state + (size_t)slot_ids[seq] * (taps - 1) * C;
+  float* state = conv_state + (size_t)slot_ids[seq] * (taps - 1) * C;
   for (int c = threadIdx.x; c < C; c += blockDim.x) {
     float xs[CONV_MAX_TAPS], ws[CONV_MAX_TAPS];
 #pragma unroll
@@ -268,6 +268,13 @@ __global__ void __launch_bounds__(1024)
     for (int j = 0; j < CONV_MAX_TAPS; ++j) acc = fmaf(ws[j], xs[j], acc);
     if (add_input) acc += x[(size_t)t * ld + c];
     o[c] = from_f32<T>(acc);
+    if (move_state) {
+      // every sequence brings one token (have == 0): xs[0 .. taps - 2] are the channel's old entries, all read above by
+      // this thread, which is their only reader in the step; the new ones are the old ones moved up and the token's own
+#pragma unroll
+      for (int j = 0; j < CONV_MAX_TAPS - 1; ++j)
+        if (j < taps - 1) state[(size_t)j * C + c] = xs[j + 1];
+    }
   }
 }
 
@@ -358,13 +365,15 @@ __global__ void __launch_bounds__(256)
 
 extern "C" int fmsamd_short_conv(const float* x, long ld, int channels, const void* conv_w, const void* bias, int weight_dtype,
                                  int taps, float* conv_state, const int* seq_of_token, const int* slot_ids, int add_input,
-                                 void* out, int out_dtype, long ldo, int n_tokens, hipStream_t stream) {
+                                 void* out, int out_dtype, long ldo, int n_tokens, int single_tokens, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && channels > 0 && ld >= channels && ldo >= channels, "short_conv: bad sizes T=%d C=%d ld=%ld ldo=%ld",
               n_tokens, channels, ld, ldo);
   FMS_REQUIRE(taps >= 1 && taps <= CONV_MAX_TAPS, "short_conv: %d taps (1 to %d)", taps, CONV_MAX_TAPS);
   FMS_REQUIRE(taps == 1 || conv_state != nullptr, "short_conv: a convolution of %d taps needs the sequences' state", taps);
   const int threads = n_tokens <= 64 ? 1024 : 256;
+  // a step in which every sequence brings one token: the kernel that convolves also moves the state on
+  const int move_state = single_tokens && taps > 1 && n_tokens < 4 * CONV_TILE;
   if (n_tokens >= 4 * CONV_TILE) {  // many rows: tiles of rows, every input loaded once
     const bool wide = channels % 4 == 0 && ld % 4 == 0 && ((uintptr_t)x % 16) == 0;
     const int per_block = 256 * (wide ? 4 : 1);
@@ -394,7 +403,7 @@ extern "C" int fmsamd_short_conv(const float* x, long ld, int channels, const vo
   }
 #define FMS_CONV(W, T)                                                                                                     \
   short_conv_kernel<W, T><<<n_tokens, threads, 0, stream>>>(x, ld, channels, (const W*)conv_w, (const W*)bias, taps, conv_state, \
-                                                            seq_of_token, slot_ids, add_input, (T*)out, ldo)
+                                                            seq_of_token, slot_ids, add_input, (T*)out, ldo, move_state)
   if (weight_dtype == FMS_F32 && out_dtype == FMS_F32) FMS_CONV(float, float);
   else if (weight_dtype == FMS_F32 && out_dtype == FMS_BF16) FMS_CONV(float, bf16);
   else if (weight_dtype == FMS_BF16 && out_dtype == FMS_F32) FMS_CONV(bf16, float);
@@ -402,7 +411,7 @@ extern "C" int fmsamd_short_conv(const float* x, long ld, int channels, const vo
   else FMS_REQUIRE(false, "short_conv: unknown dtypes %d %d", weight_dtype, out_dtype);
 #undef FMS_CONV
   FMS_LAUNCH_CHECK("short_conv");
-  if (taps > 1) {
+  if (taps > 1 && !move_state) {
     conv_state_kernel<<<n_tokens, threads, 0, stream>>>(x, ld, taps, conv_state, seq_of_token, slot_ids, n_tokens, channels);
     FMS_LAUNCH_CHECK("conv_state");
   }

@@ -17,7 +17,7 @@ import torch  # noqa: F401  (loads libamdhip64 before our library asks for it)
 
 from . import build as _build
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
@@ -62,7 +62,7 @@ _SIGNATURES = {
     "fmsamd_moe_route_grouped": [P, L, I, I, I, P, I, I, F, P, P, P],
     "fmsamd_poly_norm": [P, L, I, F, F, F, F, F, P, I, L, I, P],
     "fmsamd_group_norm_chain": [P, P, I, P, I, I, F, P, I, I, F, P, I, P, I, I, P],
-    "fmsamd_short_conv": [P, L, I, P, P, I, I, P, P, P, I, P, I, L, I, P],
+    "fmsamd_short_conv": [P, L, I, P, P, I, I, P, P, P, I, P, I, L, I, I, P],
     "fmsamd_rglru_gates": [P, L, P, P, P, P, I, P, F, P, P, P, I, I, I, P],
     "fmsamd_rglru_scan": [P, P, P, L, I, P, P, P, P, P, I, L, I, I, P],
     "fmsamd_rglru_scan_chunk": [I, I],

@@ -715,11 +715,13 @@ CONV_MAX_TAPS = 8
 
 
 def short_conv(x: torch.Tensor, col0: int, channels: int, conv_w: torch.Tensor, bias: Optional[torch.Tensor], conv_state: Optional[torch.Tensor],
-               seq_of_token: torch.Tensor, slot_ids: torch.Tensor, out_dtype: torch.dtype, add_input: bool = False) -> torch.Tensor:
+               seq_of_token: torch.Tensor, slot_ids: torch.Tensor, out_dtype: torch.dtype, add_input: bool = False,
+               single_tokens: bool = False) -> torch.Tensor:
     """A causal convolution over time on the channels col0 .. col0 + channels of float32 rows: out[t, c] = (x[t, c] if
     add_input) + bias[c] + sum_j conv_w[c, j] x[t - taps + 1 + j, c] over the sequence's own tokens -> [T, channels] in
     out_dtype.  The inputs before the step come from conv_state [slots, taps - 1, channels] (float32; zeros before a
-    sequence's start), which is then moved on to the step's last inputs."""
+    sequence's start), which is then moved on to the step's last inputs.  single_tokens: every sequence of the step
+    brings exactly one token (a decode step); the kernel that convolves then moves the state on as well."""
     _need_cuda(x, conv_w, bias, conv_state, seq_of_token, slot_ids)
     _rows2d("x", x)
     _need_i32("seq_of_token", seq_of_token)
@@ -739,7 +741,7 @@ def short_conv(x: torch.Tensor, col0: int, channels: int, conv_w: torch.Tensor, 
     view = x[:, col0 : col0 + channels]
     check(load().fmsamd_short_conv(view.data_ptr(), x.stride(0), channels, conv_w.data_ptr(), _ptr(bias), _code(conv_w.dtype), taps,
                                    _ptr(conv_state), seq_of_token.data_ptr(), slot_ids.data_ptr(), int(bool(add_input)), out.data_ptr(),
-                                   _code(out_dtype), out.stride(0), T, _stream()))
+                                   _code(out_dtype), out.stride(0), T, int(bool(single_tokens)), _stream()))
     return out
 
 

@@ -186,7 +186,7 @@ class PostNormBlock(Part):
         if self.input_taps:
             x = stream.rows(torch.float32)
             h = ops.short_conv(x, 0, self.width, self.w[self._conv_name], None, cache.state.get("block.conv"), batch.seq_of_token,
-                               batch.slot_ids, act_dtype, add_input=True)
+                               batch.slot_ids, act_dtype, add_input=True, single_tokens=batch.is_decode)
         else:
             h = stream.rows(act_dtype)
         stream.add_branch(self.mixer.forward(h, batch, cache), post_norm=self.norm1)

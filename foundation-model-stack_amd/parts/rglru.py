@@ -77,7 +77,7 @@ class RecurrentGatedUnit(Mixer):
         # the gates and the recurrence are formed from the float32 sums of this product
         proj = self.in_proj.forward(x, out_dtype=torch.float32)
         u = ops.short_conv(proj, C, C, self.w["conv.weight"], self.w["conv.bias"], state.get("conv"), batch.seq_of_token,
-                           batch.slot_ids, torch.float32)
+                           batch.slot_ids, torch.float32, single_tokens=batch.is_decode)
         a, b = ops.rglru_gates(u, self._ra_t, self._ra_b, self._ri_t, self._ri_b, self._lam, self.decay_constant, batch.seq_of_token)
         mixed = ops.rglru_scan(a, b, proj[:, :C], self.activation, state["S"], batch.seq_starts, batch.seq_of_token, batch.slot_ids,
                                batch.n_seqs, x.dtype, zero_rows=batch.is_decode)

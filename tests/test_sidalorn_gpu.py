@@ -342,14 +342,14 @@ def test_convolution_over_time_in_long_steps(lib, out_dtype, sizes):
             + (x[:, 4 : 4 + C] if add_input else 0) for x in xs]
     slots = [5, 0, 3, 7, 1, 6, 2]
 
-    def run(state, steps):
+    def run(state, steps, single_tokens=False):
         got = [[] for _ in lens]
         for lo, hi in steps:
             ns = [min(hi, len(x)) - lo for x in xs]
             keep = [j for j, n in enumerate(ns) if n > 0]
             x = torch.cat([xs[j][lo : lo + ns[j]] for j in keep]).to(DEV)
             out = ops.short_conv(x, 4, C, w.to(DEV), None if bias is None else bias.to(DEV), state, _i32([i for i, j in enumerate(keep) for _ in range(ns[j])]),
-                                 _i32([slots[j] for j in keep]), out_dtype, add_input=add_input)
+                                 _i32([slots[j] for j in keep]), out_dtype, add_input=add_input, single_tokens=single_tokens)
             at = 0
             for j in keep:
                 got[j].append(out[at : at + ns[j]].float().cpu())
@@ -366,8 +366,13 @@ def test_convolution_over_time_in_long_steps(lib, out_dtype, sizes):
     one_by_one = run(one_by_one_state, [(t, t + 1) for t in range(202)])
     for j in range(len(lens)):
         assert torch.equal(long_steps[j], one_by_one[j])
+    # the same steps announced as steps of single tokens (decode steps): one kernel convolves and moves the state on
+    fused_state = new_state()
+    fused = run(fused_state, [(t, t + 1) for t in range(202)], single_tokens=True)
+    for j in range(len(lens)):
+        assert torch.equal(fused[j], one_by_one[j])
     if taps > 1:
-        assert torch.equal(state, one_by_one_state)
+        assert torch.equal(state, one_by_one_state) and torch.equal(state, fused_state)
         torch.testing.assert_close(state[1].cpu(), xs[4][-(taps - 1):, 4 : 4 + C])
 
 
