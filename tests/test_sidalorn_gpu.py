@@ -835,6 +835,34 @@ def test_ragged_batches_with_pages_and_slots_used_again(lib, folders, name, dtyp
     assert engine.cache.n_free_slots == 3 and all(g.pool.n_held == 0 for g in engine.cache.groups)
 
 
+@pytest.mark.parametrize("name", ["A", "C"])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_prompts_together(lib, folders, name, dtype):
+    """Three long prompts in one step (the recurrence walks the step in chunks of rows that hold the borders between
+    the sequences, the convolutions in tiles), then decoded together: every request equals itself alone."""
+    from fms_amd.engine import Engine
+
+    reqs = [expected_for(folders, name, n, seed, dtype) for n, seed in ((330, 11), (150, 12), (290, 13))]
+    model = get(lib, folders, name, dtype)
+    engine = Engine(model, max_tokens=64 * 16, max_slots=3)
+    slots = [engine.new_sequence() for _ in reqs]
+    cut = [len(ids) - 6 for ids, _ in reqs]
+    out = engine.step(slots, [ids[:c] for (ids, _), c in zip(reqs, cut)], "all")
+    got, at = [], 0
+    for c in cut:
+        got.append([out[at : at + c]])
+        at += c
+    for i in range(6):
+        out = engine.step(slots, [[ids[c + i]] for (ids, _), c in zip(reqs, cut)], "last")
+        for b in range(len(reqs)):
+            got[b].append(out[b : b + 1])
+    for b, (ids, want) in enumerate(reqs):
+        judge(torch.cat(got[b]), want, dtype)
+    for s in slots:
+        engine.end_sequence(s)
+    engine.cache.check()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_a_far_key_decides_in_prompts_and_in_decoding(lib, dtype, tmp_path):
     """Queries scaled up: single keys hold most of a query's weight, many of them hundreds of tokens back and on
