@@ -373,8 +373,9 @@ extern "C" int fmsamd_short_conv(const float* x, long ld, int channels, const vo
   FMS_REQUIRE(taps == 1 || conv_state != nullptr, "short_conv: a convolution of %d taps needs the sequences' state", taps);
   const int threads = n_tokens <= 64 ? 1024 : 256;
   // a step in which every sequence brings one token: the kernel that convolves also moves the state on
-  const int move_state = single_tokens && taps > 1 && n_tokens < 4 * CONV_TILE;
-  if (n_tokens >= 4 * CONV_TILE) {  // many rows: tiles of rows, every input loaded once
+  // (of any number of sequences: a tile of rows would walk 16 sequences one after the other, each with its own state)
+  const int move_state = single_tokens && taps > 1;
+  if (n_tokens >= 4 * CONV_TILE && !single_tokens) {  // many rows: tiles of rows, every input loaded once
     const bool wide = channels % 4 == 0 && ld % 4 == 0 && ((uintptr_t)x % 16) == 0;
     const int per_block = 256 * (wide ? 4 : 1);
     const dim3 grid(ceil_div(n_tokens, CONV_TILE), ceil_div(channels, per_block));

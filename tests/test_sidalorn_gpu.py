@@ -376,6 +376,30 @@ def test_convolution_over_time_in_long_steps(lib, out_dtype, sizes):
         torch.testing.assert_close(state[1].cpu(), xs[4][-(taps - 1):, 4 : 4 + C])
 
 
+@pytest.mark.parametrize("taps", [2, 4, 7])
+def test_convolution_over_time_in_decode_steps_of_many_sequences(lib, taps):
+    """80 sequences that bring one token a step: announced as such (one kernel, which also moves the state on) and not
+    (tiles of rows, then the state's kernel): the same numbers, the plain implementation's."""
+    from fms_amd.kernels import ops
+
+    n_seq, steps, C = 80, 6, 72
+    gen = torch.Generator().manual_seed(taps)
+    x = torch.randn(n_seq, steps, C, generator=gen)
+    w, bias = torch.randn(C, taps, generator=gen), torch.randn(C, generator=gen)
+    want = torch.stack([S.convolution_over_time(x[b].double(), w.double(), bias.double()).float() for b in range(n_seq)])
+    slots = torch.randperm(100, generator=gen)[:n_seq].tolist()
+    outs, states = [], []
+    for single in (True, False):
+        state = torch.zeros(100, taps - 1, C, device=DEV)
+        got = [ops.short_conv(x[:, i].contiguous().to(DEV), 0, C, w.to(DEV), bias.to(DEV), state, _i32(list(range(n_seq))), _i32(slots),
+                              torch.float32, single_tokens=single).cpu() for i in range(steps)]
+        outs.append(torch.stack(got, dim=1))
+        states.append(state.cpu())
+    torch.testing.assert_close(outs[0], want, atol=1e-5, rtol=1e-5)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(states[0], states[1])
+    torch.testing.assert_close(states[0][slots[3]], x[3, -(taps - 1):])
+
+
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
 # the last three: steps of many tokens and blocks too wide for the kernel of small steps (the tiled kernel runs)
 @pytest.mark.parametrize("sizes", [(12, 3, 5), (60, 5, 19), (128, 1, 8), (384, 3, 33), (64, 64, 7), (1024, 2, 3), (64, 2, 4100), (2048, 1, 9),
