@@ -606,7 +606,7 @@ def test_experts_without_gates_identity_experts_and_their_sum(lib, dtype, sizes)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(3, 24), (4, 40), (8, 128), (2, 64), (5, 100), (16, 512)])
+@pytest.mark.parametrize("sizes", [(3, 24), (4, 40), (8, 128), (2, 64), (5, 100), (16, 512), (4, 256), (20, 96), (6, 384)])
 def test_attention_without_positions_over_a_latent_cache(lib, dtype, sizes):
     """No rotated part at all: two sequences whose pages lie mixed in the pool, queries at page borders and far apart,
     a sink that matters, and one query and one far key scaled so that the far key decides."""
