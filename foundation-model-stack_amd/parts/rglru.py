@@ -10,7 +10,8 @@ inside each, two square matrices make the gates,
 
 and the block's output is W_o (S * y).  What a sequence carries from token to token is S (float32) and the last
 `conv - 1` inputs of the convolution; both are fixed-size state of its slot, so whole prompts, portions of prompts and
-single tokens run the same kernels and differ by rounding only.  Everything behind the projection is float32.
+single tokens start from the same numbers and differ by rounding only (long steps walk the recurrence in chunks of rows
+side by side, which adds in another order).  Everything behind the projection is float32.
 """
 
 from __future__ import annotations
