@@ -71,6 +71,7 @@ def main() -> int:
     ap.add_argument("--max_new_tokens", type=int, default=None, help="the same as --steps: decode steps that are timed")
     ap.add_argument("--zodolorn", action="store_true",
                     help="another workload: Zodolorn beside Llama at equal layer sizes, with every kernel class's distance from its roofline")
+    ap.add_argument("--basopel", action="store_true", help="another workload: Basopel beside Llama at equal layer sizes, likewise")
     ap.add_argument("--defapel", action="store_true", help="another workload: Defapel beside Llama at equal layer sizes, likewise")
     ap.add_argument("--sidalorn", action="store_true", help="another workload: Sidalorn beside Zodolorn at equal layer sizes, likewise")
     args = ap.parse_args()
@@ -84,8 +85,8 @@ def main() -> int:
         print(f"bench.py measures one GPU: this library runs on a single MI355X, --gpus {args.gpus} is not supported")
         return 2
 
-    if args.zodolorn or args.defapel or args.sidalorn:
-        return design_comparison(args, "zodolorn" if args.zodolorn else ("defapel" if args.defapel else "sidalorn"))
+    if args.zodolorn or args.defapel or args.sidalorn or args.basopel:
+        return design_comparison(args, "zodolorn" if args.zodolorn else ("defapel" if args.defapel else ("sidalorn" if args.sidalorn else "basopel")))
 
     import torch
 
@@ -335,6 +336,14 @@ SIDALORN_SIZES = [
 ]
 
 
+# (name, width, layer pattern (c: attention in chunks, w: windowed with a distance bias, l: latent), heads, kv heads, head size,
+#  feed-forward, chunk = window, latent size, vocabulary)
+BASOPEL_SIZES = [
+    ("w2048", 2048, "ccwl", 16, 4, 128, 8192, 1024, 512, 32768),
+    ("w4096", 4096, "ccwl", 32, 8, 128, 12288, 1024, 512, 32768),
+]
+
+
 def design_comparison(args, design) -> int:
     import torch
 
@@ -355,6 +364,23 @@ def design_comparison(args, design) -> int:
     # come from memory at least once (a prompt's keys serve all its queries; a decode step reads every context once)
     state = {"keys_read": 0, "keys_loaded": 0}
 
+    def keys_of_call(a, kw):
+        """(keys read, keys loaded) of one attention call, from the step's token runs (state["runs"]: first position and
+        count per sequence, when the workload sets them) and the call's own mask: a window (a[10]), kept first keys, chunks."""
+        runs = state.get("runs")
+        if not runs:
+            return state["keys_read"], state["keys_loaded"]
+        window, chunk, keep = int(a[10]) if len(a) > 10 else 0, int(kw.get("chunk", 0) or 0), int(kw.get("keep_first", 0) or 0)
+
+        def seen(p):
+            if chunk:
+                return p % chunk + 1
+            return min(p + 1, window + min(keep, max(0, p + 1 - window))) if window else p + 1
+
+        read = sum(seen(p) for first, count in runs for p in range(first, first + count))
+        loaded = sum(max(seen(first + count - 1), min(first + count, count + seen(first) - 1)) for first, count in runs)
+        return read, loaded
+
     def nbytes(*tensors):
         return sum(t.numel() * t.element_size() for t in tensors if t is not None)
 
@@ -367,7 +393,8 @@ def design_comparison(args, design) -> int:
             return nbytes(w) + 2 * x.shape[0] * w.shape[0] * (w.shape[1] + w.shape[2]), 2.0 * x.shape[0] * w.numel()
         if name == "attention":  # grouped-query attention over keys and values of kvheads x head_dim
             H, K, D = a[6], a[7], a[8]
-            return 2 * state["keys_loaded"] * 2 * K * D + 2 * nbytes(a[0][:, : H * D]), 4.0 * state["keys_read"] * H * D
+            read, loaded = keys_of_call(a, kw)
+            return 2 * loaded * 2 * K * D + 2 * nbytes(a[0][:, : H * D]), 4.0 * read * H * D
         if name == "delta_rule":  # state read and written once a sequence; per token and head 4 passes over dim x vdim in float32
             qkv, st, n_seqs, H, D, V = a[0], a[4], a[8], a[9], a[11], a[12]
             vector_flops = 8.0 * qkv.shape[0] * H * D * V
@@ -375,7 +402,8 @@ def design_comparison(args, design) -> int:
             return nbytes(qkv, a[1], a[2], out) + 2 * n_seqs * (st.numel() // st.shape[0]) * 4, vector_flops * mfma_flops / PEAK_FLOPS["fp32"]
         if name == "latent_attention":  # one row of rank + rot a key, and the latent once more as values
             H, R, P = a[6], a[7], a[8]
-            return 2 * state["keys_loaded"] * (2 * R + P) + nbytes(a[0]) + 2 * a[0].shape[0] * H * R, 2.0 * state["keys_read"] * H * (2 * R + P)
+            read, loaded = keys_of_call(a, kw)
+            return 2 * loaded * (2 * R + P) + nbytes(a[0]) + 2 * a[0].shape[0] * H * R, 2.0 * read * H * (2 * R + P)
         if name == "rglru_gates":  # two block-diagonal products on the float32 vector units, priced like the delta rule's passes
             u, ra = a[0], a[1]
             vector_flops = 4.0 * u.shape[0] * ra.numel()
@@ -395,10 +423,10 @@ def design_comparison(args, design) -> int:
 
     watched = ["linear", "gated_linear", "linear_into_stream", "headwise_linear", "attention", "latent_attention", "moe_experts",
                "moe_route", "moe_combine", "add_norm", "norm_add_norm", "rms_norm_cols", "rope_kv_write", "qkv_rope_write",
-               "latent_kv_write", "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed",
+               "latent_kv_write", "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed", "norm_add_norm_affine",
                "delta_rule", "delta_prepare", "gated_head_norm", "qk_projection_norm", "gate_mul", "scale_", "cast", "cast_cols",
                "rglru_gates", "rglru_scan", "short_conv", "group_norm_chain", "poly_norm", "moe_route_grouped"]
-    small = {"moe_route", "moe_combine", "add_norm", "norm_add_norm", "rms_norm_cols", "rope_kv_write", "latent_kv_write",
+    small = {"moe_route", "moe_combine", "add_norm", "norm_add_norm", "norm_add_norm_affine", "rms_norm_cols", "rope_kv_write", "latent_kv_write",
              "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed", "delta_prepare", "gated_head_norm",
              "qk_projection_norm", "gate_mul", "scale_", "cast", "cast_cols", "short_conv", "group_norm_chain", "poly_norm",
              "moe_route_grouped"}
@@ -433,8 +461,9 @@ def design_comparison(args, design) -> int:
             out[kind] = (ms + first.elapsed_time(last), ideal + 1000 * max(b / read_bps, f / mfma_flops))
         return {k: {"ms": round(ms, 4), "x_roofline": round(ms / ideal, 2) if ideal else None} for k, (ms, ideal) in sorted(out.items())}
 
-    def measure(model, vocab, window=0):
-        """window: the most keys a query of the model's attention sees (0: all before it), for the attention's flops."""
+    def measure(model, vocab, window=0, per_call_masks=False):
+        """window: the most keys a query of the model's attention sees (0: all before it), for the attention's flops.
+        per_call_masks: the layers' masks differ, so every attention call is priced by its own (keys_of_call)."""
         def keys_seen(lengths):
             return sum(min(n, window) if window else n for n in lengths)
 
@@ -456,7 +485,7 @@ def design_comparison(args, design) -> int:
             out[f"prefill_{n}_ms"] = round(1000 * t, 3)
             if n == 2048:
                 slot = engine.new_sequence()
-                state.update(keys_read=keys_seen(range(1, n + 1)), keys_loaded=n)
+                state.update(keys_read=keys_seen(range(1, n + 1)), keys_loaded=n, runs=[(0, n)] if per_call_masks else None)
                 out["prefill_2048_kernels"] = classes_of_a_step(lambda: engine.step([slot], [ids], "last"))
                 engine.end_sequence(slot)
             del engine
@@ -490,7 +519,7 @@ def design_comparison(args, design) -> int:
             out[f"{name}_ms"] = round(1000 * dt / steps, 3)
             if (batch, prompt) in ((8, 1024), (8, 7000)):
                 now = [n + warmup + steps + 1 for n in lens]
-                state.update(keys_read=keys_seen(now), keys_loaded=keys_seen(now))
+                state.update(keys_read=keys_seen(now), keys_loaded=keys_seen(now), runs=[(m - 1, 1) for m in now] if per_call_masks else None)
                 out[f"{name}_kernels"] = classes_of_a_step(lambda: engine.step(slots, [[t] for t in tokens], "last"))
             for s in slots:
                 engine.end_sequence(s)
@@ -501,6 +530,30 @@ def design_comparison(args, design) -> int:
     record = {"workload": f"{design} beside {'zodolorn' if design == 'sidalorn' else 'llama'} at equal layer sizes", "layers": layers, "dtype": "bf16",
               "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
               "peak_measured": {"read_gbs": round(read_bps / 1e9, 1), "mfma_tflops": round(mfma_flops / 1e12, 1)}, "sizes": {}}
+    if design == "basopel":
+        from fms_amd.architectures.basopel import make_config as make_basopel
+
+        for name, width, pattern, heads, kv, dim, ff, span, kv_rank, vocab in BASOPEL_SIZES:
+            pattern = (pattern * layers)[:layers]
+            config = make_basopel(width=width, vocab=vocab, pattern=pattern, heads=heads, kv_heads=kv, dim=dim, vdim=dim, ff=ff, chunk=span,
+                                  window=span, latent_window=span, kv_rank=kv_rank, latent_rot=64, rot_dims=dim // 2, rot_factor=4.0,
+                                  max_positions=context)
+            model = fms_amd.from_config(config, "basopel", data_type="bf16", random_seed=args.seed)
+            mine = measure(model, vocab, per_call_masks=True)
+            del model
+            torch.cuda.empty_cache()
+            # Llama of the same width, depth, heads and gated feed-forward (its attention sees every earlier key)
+            llama = fms_amd.get_model("llama", "micro", data_type="bf16", random_seed=args.seed, emb_dim=width, nheads=heads, kvheads=kv,
+                                      nlayers=layers, hidden_dim=ff, src_vocab_size=vocab, max_expected_seq_len=context)
+            theirs = measure(llama, vocab, per_call_masks=True)
+            del llama
+            torch.cuda.empty_cache()
+            record["sizes"][name] = {"basopel": dict(config=dict(width=width, pattern=pattern, heads=heads, kv_heads=kv, dim=dim, ff=ff,
+                                                                   chunk=span, window=span, kv_rank=kv_rank, vocab=vocab), **mine),
+                                     "llama": dict(config=dict(width=width, heads=heads, kvheads=kv, head_dim=width // heads, hidden=ff,
+                                                               vocab=vocab), **theirs)}
+        print(json.dumps(record))
+        return 0
     if design == "defapel":
         from fms_amd.architectures.defapel import make_config as make_defapel
 

@@ -5,11 +5,11 @@ generation loop.  Importing the package touches no GPU; the kernel library is co
 
 from . import architectures as _architectures  # noqa: F401  (fills the registries)
 from .architectures import list_models, list_variants, register_architecture, register_model
-from .config import DefapelConfig, LLaMAConfig, ModelConfig, SidalornConfig, ZodolornConfig
+from .config import BasopelConfig, DefapelConfig, LLaMAConfig, ModelConfig, SidalornConfig, ZodolornConfig
 from .models import LLaMA, from_config, get_model, write_model_folder
 
 __all__ = [
-    "LLaMA", "LLaMAConfig", "ModelConfig", "ZodolornConfig", "DefapelConfig", "SidalornConfig", "from_config", "get_model", "write_model_folder", "list_models", "list_variants",
+    "LLaMA", "LLaMAConfig", "ModelConfig", "ZodolornConfig", "DefapelConfig", "SidalornConfig", "BasopelConfig", "from_config", "get_model", "write_model_folder", "list_models", "list_variants",
     "register_architecture", "register_model", "generate", "generate_requests", "pad_input_ids", "Engine",
 ]
 

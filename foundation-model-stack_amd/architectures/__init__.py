@@ -1,4 +1,4 @@
-from . import defapel, llama, sidalorn, zodolorn  # noqa: F401  (register the architectures, their adapters and variants)
+from . import basopel, defapel, llama, sidalorn, zodolorn  # noqa: F401  (register the architectures, their adapters and variants)
 from .registry import (
     Architecture,
     architecture_for_hf,

@@ -38,6 +38,12 @@ class KVNeed:
     # or a function of what it keeps as keys, like attention over a latent)
     values: bool = True
     value_dim: int = 0  # size of a value if it is not head_dim (0: head_dim)
+    # with a window: the sequence's first keep_first keys stay visible to every later query (their pages are never
+    # given back)
+    keep_first: int = 0
+    # c > 0: positions are cut into chunks of c, counted from the sequence's start, and a query sees the keys of its own
+    # chunk only (pages before the chunk of a step's first query are given back)
+    chunk: int = 0
 
 
 @dataclasses.dataclass(frozen=True)
@@ -56,9 +62,12 @@ class KVGroup:
         self.values: Optional[torch.Tensor] = None
         # slot -> logical page list; -1 marks a page given back because the window has passed it
         self.pages: Dict[int, List[int]] = {}
-        # slot -> index of the slot's first page that has not been given back (everything before it is -1): a
-        # window's releases are looked for from there, not from the sequence's start, at every step
+        # slot -> index of the slot's first page that has not been given back (everything before it is -1, but for the
+        # `kept` pages at the sequence's start, which stay): a window's releases are looked for from there, not from
+        # the sequence's start, at every step
         self.first_held: Dict[int, int] = {}
+        # pages at a sequence's start that a window never gives back (they hold the first tokens that stay visible)
+        self.kept = pages_for(need.keep_first) if (need.window > 0 and need.keep_first > 0) else 0
 
     def allocate_storage(self, dtype: torch.dtype, device) -> None:
         n, K, D = self.pool.n_pages, self.need.kv_heads, self.need.head_dim
@@ -187,9 +196,13 @@ class SequenceCache:
         for group in self.groups:
             pages = group.pages[slot]
             release = []
-            if group.need.window > 0:
+            first_visible = 0
+            if group.need.chunk > 0:
+                first_visible = start - start % group.need.chunk
+            elif group.need.window > 0:
                 first_visible = max(0, start - group.need.window + 1)
-                release = list(range(group.first_held[slot], min(first_visible // PAGE_TOKENS, len(pages))))
+            if first_visible > 0:
+                release = list(range(max(group.first_held[slot], group.kept), min(first_visible // PAGE_TOKENS, len(pages))))
             plans.append((group, release, max(0, pages_for(new_len) - len(pages))))
         return plans
 
@@ -243,7 +256,7 @@ class SequenceCache:
     def pages_held(self, slot: int) -> int:
         """How many pages the slot holds over all groups: it changes when the sequence gets a page and when a
         window gives one back, so whoever keeps a copy of the block tables knows when to read them again."""
-        return sum(len(group.pages[slot]) - group.first_held[slot] for group in self.groups)
+        return sum(len(group.pages[slot]) - max(0, group.first_held[slot] - group.kept) for group in self.groups)
 
     def block_table(self, group_index: int, slots: Sequence[int], n_columns: Optional[int] = None) -> torch.Tensor:
         """int32 [len(slots), n_columns] page numbers on the host (unused entries and released pages: -1)."""
@@ -289,5 +302,6 @@ class SequenceCache:
                 raise AssertionError("page lists and live slots differ")
             for slot, pages in group.pages.items():
                 first = group.first_held[slot]
-                if any(p >= 0 for p in pages[:first]) or any(p < 0 for p in pages[first:]):
-                    raise AssertionError("released pages are not exactly the pages before the first held one")
+                gone = set(range(group.kept, first))
+                if any((p < 0) != (i in gone) for i, p in enumerate(pages)):
+                    raise AssertionError("released pages are not exactly the pages between the kept ones and the first held one")

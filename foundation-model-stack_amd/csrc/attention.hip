@@ -21,16 +21,27 @@
 // ==========================================================================
 #define GEN_THREADS 256
 
+// Which keys a query at position pos sees, beside j <= pos: a sliding window (the last `window` keys; 0: all), of which the
+// sequence's first `keep_first` keys are exempt; or chunks (positions cut into runs of `chunk`, counted from the sequence's
+// start; a query sees its own run only).  lower_bound is the first key of the contiguous run that ends at pos.
+__device__ __forceinline__ int lower_bound(int pos, int window, int chunk) {
+  if (chunk > 0) return pos - pos % chunk;
+  return (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+}
+
 // TERMS: the scores carry further terms (fms/modules/positions.py:9-36, the reference's adjusted_mask): a soft cap
-// cap * tanh(score / cap), and a bias slope[head] * (key position - query position), which is zero or negative.
-// Without TERMS neither is compiled in.
+// cap * tanh(score / cap); a bias slope[head] * (key position - query position), which is zero or negative; a learned
+// bias by distance, dist_bias[head][min(pos - j, dist_len - 1)] (the host has turned distances into the table's rows);
+// a sink, one logit per head that takes part in the softmax's denominator and has neither key nor value.
+// Without TERMS none of them is compiled in.
 template <typename T, bool TERMS>
 __global__ void __launch_bounds__(GEN_THREADS)
     attn_generic_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out, long out_stride,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                         const int* __restrict__ block_table, int table_stride, const T* __restrict__ k_cache,
                         const T* __restrict__ v_cache, int nheads, int kvheads, int head_dim, int vdim, float scale, int window,
-                        const float* __restrict__ slopes, float soft_cap) {
+                        const float* __restrict__ slopes, float soft_cap, int chunk, int keep_first,
+                        const float* __restrict__ sink, const float* __restrict__ dist_bias, int dist_len) {
   __shared__ float qs[256];
   __shared__ float ps[GEN_THREADS];
   __shared__ float scratch[17];
@@ -43,7 +54,10 @@ __global__ void __launch_bounds__(GEN_THREADS)
     return;
   }
   const int pos = positions[t];
-  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  const int lo = lower_bound(pos, window, TERMS ? chunk : 0);
+  // the keys a query sees, counted through: first the kept keys in front of the window, then lo .. pos
+  const int n_kept = TERMS ? (keep_first < lo ? keep_first : lo) : 0;
+  const int n_keys = n_kept + pos - lo + 1;
   const int kh = h / (nheads / kvheads);
   const int* bt = block_table + (size_t)seq * table_stride;
   const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
@@ -54,10 +68,12 @@ __global__ void __launch_bounds__(GEN_THREADS)
   __syncthreads();
 
   float m_run = -1e30f, l_run = 0.f, acc = 0.f;  // acc: this thread's output element d = threadIdx.x
-  for (int base = lo; base <= pos; base += GEN_THREADS) {
-    const int j = base + threadIdx.x;
+  if (TERMS && sink != nullptr) m_run = sink[h], l_run = 1.f;  // the sink: a weight of exp(sink - maximum) from the start
+  for (int base = 0; base < n_keys; base += GEN_THREADS) {
+    const int u = base + threadIdx.x;
+    const int j = u < n_kept ? u : lo + (u - n_kept);
     float s = -INFINITY;
-    if (j <= pos) {
+    if (u < n_keys) {
       const T* krow = k_cache + readable_page(bt[j / PAGE_TOKENS]) * page_elems +
                       ((size_t)kh * PAGE_TOKENS + j % PAGE_TOKENS) * head_dim;
       float dot = 0.f;
@@ -66,10 +82,11 @@ __global__ void __launch_bounds__(GEN_THREADS)
       if (TERMS) {
         if (soft_cap > 0.f) s = soft_cap * tanhf(s / soft_cap);
         if (slopes != nullptr) s = fmaf(slopes[h], (float)(j - pos), s);
+        if (dist_bias != nullptr) s += dist_bias[(size_t)h * dist_len + (pos - j < dist_len ? pos - j : dist_len - 1)];
       }
     }
     const float m_new = fmaxf(m_run, block_max(s, scratch));
-    const float p = j <= pos ? expf(s - m_new) : 0.f;
+    const float p = u < n_keys ? expf(s - m_new) : 0.f;
     const float alpha = expf(m_run - m_new);
     ps[threadIdx.x] = p;
     const float psum = block_sum(p, scratch);  // has the barriers that publish ps
@@ -78,9 +95,10 @@ __global__ void __launch_bounds__(GEN_THREADS)
     if ((int)threadIdx.x < vdim) {
       const int d = threadIdx.x;
       float a = acc * alpha;
-      const int n = pos - base + 1 < GEN_THREADS ? pos - base + 1 : GEN_THREADS;
+      const int n = n_keys - base < GEN_THREADS ? n_keys - base : GEN_THREADS;
       for (int i = 0; i < n; ++i) {
-        const int jj = base + i;
+        const int uu = base + i;
+        const int jj = uu < n_kept ? uu : lo + (uu - n_kept);
         const T* vrow = v_cache + readable_page(bt[jj / PAGE_TOKENS]) * vpage_elems +
                         ((size_t)kh * vdim + d) * PAGE_TOKENS + jj % PAGE_TOKENS;
         a = fmaf(ps[i], to_f32(*vrow), a);
@@ -339,7 +357,7 @@ __global__ void __launch_bounds__(WAVES* WAVE)
                              const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
                              const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                              const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
-                             int window, float soft_cap) {
+                             int window, float soft_cap, int chunk, const float* __restrict__ sink) {
   static_assert(WAVES * QT * 16 == PREFILL_QBLOCK, "a block covers PREFILL_QBLOCK tokens");
   const int h = blockIdx.y;
   const int wave = threadIdx.x / WAVE;
@@ -365,21 +383,21 @@ __global__ void __launch_bounds__(WAVES* WAVE)
     const bool valid = t < t_end;
     load_query<MAXDT>(qreg[qt], valid ? q + (size_t)t * q_stride + (size_t)h * head_dim : nullptr, head_dim);
     qpos[qt] = valid ? positions[t] : -1;
-    qlo[qt] = (valid && window > 0 && qpos[qt] - window + 1 > 0) ? qpos[qt] - window + 1 : 0;
+    qlo[qt] = valid ? lower_bound(qpos[qt], window, chunk) : 0;
   }
   // key range of the wave: tokens of a block are consecutive positions of one sequence
   {
     const int t_last = (t0 + QT * 16 < t_end ? t0 + QT * 16 : t_end) - 1;
     key_hi = positions[t_last];
     const int first = positions[t0];
-    key_lo = (window > 0 && first - window + 1 > 0) ? first - window + 1 : 0;
+    key_lo = lower_bound(first, window, chunk);
   }
 
   WaveState<MAXDT, QT> st;
   wave_state_init(st);
   // every column sees the keys from the last token's window start up to the first token's position
   const int full_hi = positions[t0];
-  const int full_lo = (window > 0 && key_hi - window + 1 > 0) ? key_hi - window + 1 : 0;
+  const int full_lo = lower_bound(key_hi, window, chunk);
   attn_wave_pages<MAXDT, QT>(st, qreg, qpos, qlo, key_lo, key_hi, key_lo / PAGE_TOKENS, 1, bt, k_cache, v_cache,
                              page_elems, kh, head_dim, make_scale2(scale, soft_cap), full_lo, full_hi);
 
@@ -389,6 +407,7 @@ __global__ void __launch_bounds__(WAVES* WAVE)
     float l = st.l[qt];
     l += __shfl_xor(l, 16, WAVE);
     l += __shfl_xor(l, 32, WAVE);
+    if (sink != nullptr) l += __builtin_amdgcn_exp2f(sink[h] * LOG2E - st.m[qt]);  // the sink counts once a column
     const int t = t0 + qt * 16 + r;
     if (t < t_end) {
       const float inv = l > 0.f ? 1.f / l : 0.f;
@@ -425,7 +444,8 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
                             const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
                             int n_qblocks, const int* __restrict__ block_table, int table_stride,
                             const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, int nheads,
-                            int kvheads, int head_dim_arg, float scale, int window, int hb, float soft_cap) {
+                            int kvheads, int head_dim_arg, float scale, int window, int hb, float soft_cap, int chunk,
+                            const float* __restrict__ sink) {
   const int head_dim = EXACT ? MAXDT * 16 : head_dim_arg;
   constexpr int KS = MAXDT * 16 + LDS_PAD;    // LDS row stride of the key page [64][KS]
   constexpr int VS = PAGE_TOKENS + LDS_PAD;   // LDS row stride of the transposed value page [head_dim][VS]
@@ -474,20 +494,20 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
     const bool valid = t < t_end;
     load_query<MAXDT>(qreg[qt], valid ? q + (size_t)t * q_stride + (size_t)h * head_dim : nullptr, head_dim);
     qpos[qt] = valid ? positions[t] : -1;
-    qlo[qt] = (valid && window > 0 && qpos[qt] - window + 1 > 0) ? qpos[qt] - window + 1 : 0;
+    qlo[qt] = valid ? lower_bound(qpos[qt], window, chunk) : 0;
   }
   int wave_hi = -1, wave_lo = 0, full_hi = -1, full_lo = 0;  // keys some / every column of the wave sees
   if (has_work) {
     const int t_last = (t0 + QT * 16 < t_end ? t0 + QT * 16 : t_end) - 1;
     wave_hi = positions[t_last];
     full_hi = positions[t0];
-    wave_lo = (window > 0 && full_hi - window + 1 > 0) ? full_hi - window + 1 : 0;
-    full_lo = (window > 0 && wave_hi - window + 1 > 0) ? wave_hi - window + 1 : 0;
+    wave_lo = lower_bound(full_hi, window, chunk);
+    full_lo = lower_bound(wave_hi, window, chunk);
   }
   // the block's keys: tokens of a block are consecutive positions of one sequence
   const int blk_first = positions[t_begin];
   const int blk_hi = positions[t_end - 1];
-  const int blk_lo = (window > 0 && blk_first - window + 1 > 0) ? blk_first - window + 1 : 0;
+  const int blk_lo = lower_bound(blk_first, window, chunk);
   const int page_first = blk_lo / PAGE_TOKENS, page_last = blk_hi / PAGE_TOKENS;
 
   // cooperative copy: chunk id -> (row, 16-byte column) of the page in global memory and in LDS
@@ -573,6 +593,7 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
       float l = st.l[qt] * f0 + l1 * f1;
       l += __shfl_xor(l, 16, WAVE);
       l += __shfl_xor(l, 32, WAVE);
+      if (sink != nullptr) l += __builtin_amdgcn_exp2f(sink[h] * LOG2E - m);  // the sink counts once a column
       const int t = t0 + qt * 16 + r;
       if (t < t_end) {
         const float inv = l > 0.f ? 1.f / l : 0.f;
@@ -683,7 +704,8 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
                               const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
                               int n_qblocks, const int* __restrict__ block_table, int table_stride,
                               const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, int nheads,
-                              int kvheads, float scale, int window, int hb, float soft_cap) {
+                              int kvheads, float scale, int window, int hb, float soft_cap, int chunk,
+                              const float* __restrict__ sink) {
   constexpr int head_dim = DT32 * 32;
   constexpr int KS = head_dim + LDS_PAD;      // LDS row stride of the key page [64][KS]
   constexpr int VS = PAGE_TOKENS + LDS_PAD;   // LDS row stride of the transposed value page [head_dim][VS]
@@ -733,18 +755,18 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
     qreg[c] = v;
   }
   const int qpos = valid ? positions[t] : -1;
-  const int qlo = (valid && window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
+  const int qlo = valid ? lower_bound(qpos, window, chunk) : 0;
   int wave_hi = -1, wave_lo = 0, full_hi = -1, full_lo = 0;  // keys some / every column of the wave sees
   if (has_work) {
     const int t_last = (t0 + 32 < t_end ? t0 + 32 : t_end) - 1;
     wave_hi = positions[t_last];
     full_hi = positions[t0];
-    wave_lo = (window > 0 && full_hi - window + 1 > 0) ? full_hi - window + 1 : 0;
-    full_lo = (window > 0 && wave_hi - window + 1 > 0) ? wave_hi - window + 1 : 0;
+    wave_lo = lower_bound(full_hi, window, chunk);
+    full_lo = lower_bound(wave_hi, window, chunk);
   }
   const int blk_first = positions[t_begin];
   const int blk_hi = positions[t_end - 1];
-  const int blk_lo = (window > 0 && blk_first - window + 1 > 0) ? blk_first - window + 1 : 0;
+  const int blk_lo = lower_bound(blk_first, window, chunk);
   const int page_first = blk_lo / PAGE_TOKENS, page_last = blk_hi / PAGE_TOKENS;
 
   constexpr int PF = 2;
@@ -817,6 +839,7 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
     const float f0 = __builtin_amdgcn_exp2f(st.m - m), f1 = __builtin_amdgcn_exp2f(m1 - m);  // base-2 maxima
     float l = st.l * f0 + l1 * f1;
     l += __shfl_xor(l, 32, WAVE);
+    if (sink != nullptr) l += __builtin_amdgcn_exp2f(sink[h] * LOG2E - m);  // the sink counts once a column
     if (valid) {
       const float inv = l > 0.f ? 1.f / l : 0.f;
       bf16* orow = out + (size_t)t * out_stride + (size_t)h * head_dim;
@@ -1115,7 +1138,8 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                             const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                             const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
-                            int window, int tile_cols, const int* __restrict__ row_order, float soft_cap) {
+                            int window, int tile_cols, const int* __restrict__ row_order, float soft_cap, int chunk,
+                            const float* __restrict__ sink) {
   extern __shared__ float lds_dynamic[];  // not staged: [wave][tile_cols columns][head_dim + 2]
   __shared__ __attribute__((aligned(16))) bf16 stage[STAGED ? MAXW * 8192 : 8];
   // where the waves' partial results meet: a region of its own, or (staged) the head of each wave's page buffer
@@ -1153,7 +1177,7 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
     return;
   }
   const int pos = uniform_load(positions + t);
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = lower_bound(pos, window, chunk);
   int page_lo, page_hi;
   if (split >= split_pages(lo, pos, n_splits, split, &page_lo, &page_hi)) {
     leave_empty();
@@ -1219,6 +1243,7 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
     }
     const int head = head0 + c;
     if (n_splits == 1) {
+      if (sink != nullptr) lsum += __builtin_amdgcn_exp2f(sink[head] * LOG2E - m);  // the sink counts once
       out[(size_t)t * out_stride + (size_t)head * head_dim + d] = (bf16)(lsum > 0.f ? o / lsum : 0.f);
     } else {
       const size_t base = ((size_t)t * nheads + head) * n_splits + split;
@@ -1236,7 +1261,8 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
 // and none of them waits for index data: a split without keys carries the maximum DECODE_EMPTY, and whatever
 // its other numbers are, they are set aside (a row of which every split is empty, a padding row, becomes zeros).
 __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                         bf16* __restrict__ out, long out_stride, int nheads, int head_dim, int n_splits) {
+                                         bf16* __restrict__ out, long out_stride, int nheads, int head_dim, int n_splits,
+                                         const float* __restrict__ sink) {
   const int h = blockIdx.x;
   const int t = blockIdx.y;
   const size_t base = ((size_t)t * nheads + h) * n_splits;
@@ -1269,6 +1295,8 @@ __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const
       }
       m = m_new;
     }
+    // the sink counts once, over all splits (a row without keys, a padding row, has m = DECODE_EMPTY and becomes zeros)
+    if (sink != nullptr) l += __builtin_amdgcn_exp2f(sink[h] * LOG2E - m);
     out[(size_t)t * out_stride + (size_t)h * head_dim + d] = (bf16)(l > 0.f ? o / l : 0.f);
   }
 }
@@ -1290,7 +1318,8 @@ extern "C" int fmsamd_attn_generic(const void* q, long q_stride, void* out, long
                                    const int* positions, const int* seq_of_token, const int* block_table,
                                    int table_stride, const void* k_cache, const void* v_cache, int n_tokens,
                                    int nheads, int kvheads, int head_dim, float scale, int window,
-                                   const float* slopes, float soft_cap, int value_dim, hipStream_t stream) {
+                                   const float* slopes, float soft_cap, int value_dim, int chunk, int keep_first,
+                                   const float* sink, const float* dist_bias, int dist_len, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   const int vdim = value_dim > 0 ? value_dim : head_dim;
   if (check_common("attn_generic", n_tokens, nheads, kvheads, head_dim, q_stride, vdim == head_dim ? out_stride : q_stride)) return -1;
@@ -1298,11 +1327,15 @@ extern "C" int fmsamd_attn_generic(const void* q, long q_stride, void* out, long
   FMS_REQUIRE(n_tokens <= 65535, "attn_generic: %d tokens exceed one launch (65535)", n_tokens);
   FMS_REQUIRE(soft_cap >= 0.f, "attn_generic: soft cap %g is negative", (double)soft_cap);
   dim3 grid(nheads, n_tokens);
-  const bool terms = slopes != nullptr || soft_cap > 0.f;
+  FMS_REQUIRE(chunk >= 0 && keep_first >= 0 && !(chunk > 0 && (window > 0 || keep_first > 0)),
+              "attn_generic: chunks (%d) go with neither a window (%d) nor kept first keys (%d)", chunk, window, keep_first);
+  FMS_REQUIRE(dist_bias == nullptr || dist_len > 0, "attn_generic: a distance table needs a length");
+  const bool terms = slopes != nullptr || soft_cap > 0.f || chunk > 0 || keep_first > 0 || sink != nullptr || dist_bias != nullptr;
 #define FMS_GEN(T, TERMS)                                                                                              \
   attn_generic_kernel<T, TERMS><<<grid, GEN_THREADS, 0, stream>>>(                                                     \
       (const T*)q, q_stride, (T*)out, out_stride, positions, seq_of_token, block_table, table_stride, (const T*)k_cache, \
-      (const T*)v_cache, nheads, kvheads, head_dim, vdim, scale, window, slopes, soft_cap)
+      (const T*)v_cache, nheads, kvheads, head_dim, vdim, scale, window, slopes, soft_cap, chunk, keep_first, sink,    \
+      dist_bias, dist_len)
   if (dtype == FMS_F32) {
     if (terms)
       FMS_GEN(float, true);
@@ -1350,8 +1383,10 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
                                         const int* qblock_len, int n_qblocks, int qblock_tokens,
                                         const int* block_table, int table_stride, const void* k_cache,
                                         const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
-                                        float scale, int window, float soft_cap, hipStream_t stream) {
+                                        float scale, int window, float soft_cap, int chunk, const float* sink,
+                                        hipStream_t stream) {
   if (n_tokens == 0 || n_qblocks == 0) return 0;
+  FMS_REQUIRE(chunk >= 0 && !(chunk > 0 && window > 0), "attn_prefill_bf16: a window (%d) and chunks (%d) do not go together", window, chunk);
   if (check_common("attn_prefill_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_prefill_bf16: head size %d is no multiple of 16", head_dim);
   FMS_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0, "attn_prefill_bf16: row strides must keep 16-byte alignment");
@@ -1363,7 +1398,7 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
     dim3 grid(n_qblocks, nheads);
     attn_prefill_bf16_kernel<16, 1, 8><<<grid, dim3(8 * WAVE), 0, stream>>>(
         (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,
-        block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale, window, soft_cap);
+        block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale, window, soft_cap, chunk, sink);
     FMS_LAUNCH_CHECK("attn_prefill_bf16");
     return 0;
   }
@@ -1382,17 +1417,17 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
     attn_prefill_lds_kernel<M, LDS_QT, LDS_UNITS, true><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(          \
         (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,       \
         n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads,         \
-        head_dim, scale, window, hb, soft_cap);                                                                    \
+        head_dim, scale, window, hb, soft_cap, chunk, sink);                                                       \
   else                                                                                                             \
     attn_prefill_lds_kernel<M, LDS_QT, LDS_UNITS, false><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(         \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,         \
       n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, \
-      scale, window, hb, soft_cap);                                                                                \
+      scale, window, hb, soft_cap, chunk, sink);                                                                   \
   } while (0)
 #define FMS_PL32(D32)                                                                                              \
   attn_prefill_lds32_kernel<D32, LDS_UNITS><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(                      \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len, n_qblocks, \
-      block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, scale, window, hb, soft_cap)
+      block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, scale, window, hb, soft_cap, chunk, sink)
   if (head_dim == 128)  // head sizes with a 32x32x16 kernel of their own
     FMS_PL32(4);
   else if (head_dim == 64)
@@ -1417,8 +1452,10 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
                                        const int* block_table, int table_stride, const void* k_cache,
                                        const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
                                        float scale, int window, int max_context, int pages_per_split, int waves,
-                                       int staged, const int* row_order, float soft_cap, hipStream_t stream) {
+                                       int staged, const int* row_order, float soft_cap, int chunk, const float* sink,
+                                       hipStream_t stream) {
   if (n_tokens == 0) return 0;
+  FMS_REQUIRE(chunk >= 0 && !(chunk > 0 && window > 0), "attn_decode_bf16: a window (%d) and chunks (%d) do not go together", window, chunk);
   if (check_common("attn_decode_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_decode_bf16: head size %d is no multiple of 16", head_dim);
   FMS_REQUIRE(q_stride % 8 == 0, "attn_decode_bf16: query row stride must keep 16-byte alignment");
@@ -1444,7 +1481,7 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
   attn_decode_bf16_kernel<M, MAXW, STAGED><<<grid, dim3(waves * WAVE), LDS, stream>>>(                               \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, part_o, part_ml, n_splits, positions, seq_of_token,          \
       block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale,       \
-      window, tile_cols, row_order, soft_cap)
+      window, tile_cols, row_order, soft_cap, chunk, sink)
   FMS_REQUIRE(staged == 0 || head_dim == 128, "attn_decode_bf16: pages go through LDS for head size 128 only");
   if (staged != 0) {
     // the waves' results meet in the page buffers: 16 KB a wave hold 16 columns of 130 floats
@@ -1463,7 +1500,7 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
   if (n_splits > 1) {
     dim3 mgrid(nheads, n_tokens);
     attn_decode_merge_kernel<<<mgrid, head_dim <= 64 ? 64 : 128, 0, stream>>>(part_o, part_ml, (bf16*)out, out_stride, nheads,
-                                                                              head_dim, n_splits);
+                                                                              head_dim, n_splits, sink);
     FMS_LAUNCH_CHECK("attn_decode_merge");
   }
   return 0;

@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define FMSAMD_ABI_VERSION 7
+#define FMSAMD_ABI_VERSION 8
 
 // element types
 #define FMS_F32 0
@@ -64,13 +64,19 @@ int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const int* posit
 // causal attention over the cache; any element type, any even head size up to 256.  Further terms of the scores:
 // slopes (float32 [nheads] or null): score += slopes[head] * (key position - query position); soft_cap (0: none):
 // score = soft_cap * tanh(score / soft_cap), before the slope term.  value_dim (0: head_dim): values and output heads
-// of another size than the keys.
+// of another size than the keys.  Which keys a query sees beside the causal rule: the last `window` (0: all), of which the
+// sequence's first `keep_first` keys are exempt; or (chunk > 0, no window) the keys of the query's own run of `chunk`
+// positions, counted from the sequence's start.  sink (float32 [nheads] or null): a logit per head that joins the softmax's
+// denominator and has neither key nor value.  dist_bias (float32 [nheads, dist_len] or null): score +=
+// dist_bias[head][min(distance, dist_len - 1)], not scaled and not capped.
 int fmsamd_attn_generic(const void* q, long q_stride, void* out, long out_stride, int dtype, const int* positions,
                         const int* seq_of_token, const int* block_table, int table_stride, const void* k_cache,
                         const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim, float scale,
-                        int window, const float* slopes, float soft_cap, int value_dim, hipStream_t stream);
+                        int window, const float* slopes, float soft_cap, int value_dim, int chunk, int keep_first,
+                        const float* sink, const float* dist_bias, int dist_len, hipStream_t stream);
 
-// soft_cap (0: none) of the two bfloat16 kernels: scores become soft_cap * tanh(score / soft_cap).
+// soft_cap (0: none) of the two bfloat16 kernels: scores become soft_cap * tanh(score / soft_cap); chunk and sink as in
+// fmsamd_attn_generic.
 // bfloat16 prefill: the step is cut into query blocks of at most fmsamd_attn_prefill_qblock(...) consecutive
 // tokens of one sequence; the same number goes into the call as qblock_tokens
 int fmsamd_attn_prefill_qblock(int nheads, int kvheads, int head_dim, int n_tokens);
@@ -78,7 +84,7 @@ int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_s
                              const int* seq_of_token, const int* qblock_start, const int* qblock_len, int n_qblocks,
                              int qblock_tokens, const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
                              int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
-                             float soft_cap, hipStream_t stream);
+                             float soft_cap, int chunk, const float* sink, hipStream_t stream);
 
 // bfloat16 decode: one token per sequence.  The context bound max_context is cut into splits of
 // `pages_per_split` pages, and every sequence deals its own pages out evenly over that many blocks of `waves`
@@ -92,7 +98,7 @@ int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, long out_st
                             const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
                             int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
                             int max_context, int pages_per_split, int waves, int staged, const int* row_order,
-                            float soft_cap, hipStream_t stream);
+                            float soft_cap, int chunk, const float* sink, hipStream_t stream);
 
 // c[M, N] = a[M, K] w[N, K]^T (+ bias[N])
 int fmsamd_gemm_f32(const float* a, long lda, const float* w, const float* bias, float* c, long ldc, int M, int N,
@@ -175,6 +181,13 @@ int fmsamd_probe_mfma(int blocks, int iterations, int large, float* out, double*
 int fmsamd_norm_add_norm(float* resid, const void* branch, int act_dtype, const void* branch_weight, float branch_eps,
                          const void* weight, int weight_dtype, float eps, void* out, const int* rows, int n_out, int width,
                          hipStream_t stream);
+// The same for norms that may take the mean off and add a shift: with N(v; w, b, mean) = (v - [mean of v]) /
+// sqrt([variance or mean square of v] + eps) * w + b, resid += N(branch; branch_weight, branch_bias, branch_mean) and
+// out = N(resid; weight, bias, mean).  The four vectors have weight_dtype; any may be null.
+int fmsamd_norm_add_norm_affine(float* resid, const void* branch, int act_dtype, const void* branch_weight,
+                                const void* branch_bias, float branch_eps, int branch_mean, const void* weight,
+                                const void* bias, int weight_dtype, float eps, int use_mean, void* out, const int* rows,
+                                int n_out, int width, hipStream_t stream);
 // out[t, 0:n] = x[t, col0 : col0 + n] / rms * weight for float32 rows ldx apart
 int fmsamd_rms_norm_cols(const float* x, long ldx, int col0, int n, const void* weight, int weight_dtype, float eps,
                          void* out, int out_dtype, long ldo, int rows, hipStream_t stream);
@@ -255,13 +268,18 @@ int fmsamd_moe_route_grouped(const float* logits, long ld, int n_tokens, int n_o
 
 // ---- steps around attention (attention_extras.hip) ------------------------------------------------------------------
 // float32 rows [q (nq) | k (nk) | v (nv)]: out = [q / rms(q) * wq | k / rms(k) * wk | v], each norm over its whole run of
-// columns; rows whose seq_of_token is negative are skipped (seq_of_token null: none are)
+// columns; rows whose seq_of_token is negative are skipped (seq_of_token null: none are).  norm_dim > 0: the norms run
+// over every run of norm_dim columns (a head) by itself, with weights of norm_dim entries that all heads share.
+// v_first (rows of out's type, ld_first apart, or null) and v_lambda (one float32 number on the device): the values
+// leave as (1 - lambda) v + lambda v_first.
 int fmsamd_qk_projection_norm(const float* proj, long ld, int nq, int nk, int nv, const void* wq, const void* wk,
                               int weight_dtype, float eps, void* out, int out_dtype, long ldo, const int* seq_of_token,
-                              int n_tokens, hipStream_t stream);
-// out = x * act(gate) * scale (gate: float32 logits or null)
+                              int n_tokens, int norm_dim, const void* v_first, long ld_first, const void* v_lambda,
+                              hipStream_t stream);
+// out = x * act(gate) * scale (gate: float32 logits or null); group > 1: one gate column for every run of `group` columns
+// of x (a gate per head)
 int fmsamd_gate_mul(const void* x, long ldx, const float* gate, long ldg, int act, float scale, void* out, long ldo,
-                    int dtype, int n_tokens, int cols, hipStream_t stream);
+                    int dtype, int n_tokens, int cols, int group, hipStream_t stream);
 int fmsamd_scale_f32(float* x, long n, float s, hipStream_t stream);
 // out[t, 0:n] = x[t, 0:n] (x: float32 rows ldx apart, already offset to the first column) in out_dtype
 int fmsamd_cast_cols(const float* x, long ldx, void* out, int out_dtype, long ldo, int n_tokens, int n, hipStream_t stream);

@@ -387,3 +387,84 @@ extern "C" int fmsamd_clamped_gated_act(const void* gu, void* out, int dtype, in
   FMS_LAUNCH_CHECK("clamped_gated_act");
   return 0;
 }
+
+// --------------------------------------------------------------------------
+// The chain for norms that may take the mean off and add a shift (layer norms on both sides of a branch):
+//   stream += N(branch; wb, bb);  out = N(stream; w, b),  N(v; w, b) = (v - mean) / sqrt(var + eps) * w + b,
+// var the mean of the squared deviations (without `mean`: no mean is taken off and var is the mean square).  One block
+// per output row; the row waits in LDS between the reductions; the mean is found first and the deviations are squared
+// afterwards, so nothing is lost where the mean is large against the spread.  All float32.
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+    norm_add_norm_affine_kernel(float* __restrict__ resid, const T* __restrict__ branch, const void* __restrict__ wb,
+                                const void* __restrict__ bb, float eps_b, int mean_b, const void* __restrict__ w,
+                                const void* __restrict__ b, int w_dtype, float eps, int use_mean, T* __restrict__ out,
+                                const int* __restrict__ rows, int width) {
+  extern __shared__ float row[];
+  __shared__ float scratch[17];
+  const int r = rows ? rows[blockIdx.x] : blockIdx.x;
+  float* x = resid + (size_t)r * width;
+  const T* br = branch + (size_t)r * width;
+  const float inv_n = 1.f / (float)width;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = to_f32(br[i]);
+    row[i] = v;
+    s += v;
+  }
+  float mean = mean_b ? block_sum(s, scratch) * inv_n : 0.f;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float d = row[i] - mean;
+    sq = fmaf(d, d, sq);
+  }
+  float rs = rsqrtf(block_sum(sq, scratch) * inv_n + eps_b);
+  s = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = (row[i] - mean) * rs * load_scale(wb, w_dtype, i);
+    if (bb != nullptr) v += load_scale(bb, w_dtype, i);
+    v += x[i];
+    row[i] = v;
+    if (!rows) x[i] = v;
+    s += v;
+  }
+  if (out == nullptr) return;
+  mean = use_mean ? block_sum(s, scratch) * inv_n : 0.f;
+  sq = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float d = row[i] - mean;
+    sq = fmaf(d, d, sq);
+  }
+  rs = rsqrtf(block_sum(sq, scratch) * inv_n + eps);
+  T* o = out + (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = (row[i] - mean) * rs * load_scale(w, w_dtype, i);
+    if (b != nullptr) v += load_scale(b, w_dtype, i);
+    o[i] = from_f32<T>(v);
+  }
+}
+
+extern "C" int fmsamd_norm_add_norm_affine(float* resid, const void* branch, int act_dtype, const void* branch_weight,
+                                           const void* branch_bias, float branch_eps, int branch_mean, const void* weight,
+                                           const void* bias, int weight_dtype, float eps, int use_mean, void* out,
+                                           const int* rows, int n_out, int width, hipStream_t stream) {
+  if (n_out == 0) return 0;
+  FMS_REQUIRE(n_out > 0 && width > 0 && width <= 16384, "norm_add_norm_affine: bad sizes rows=%d width=%d", n_out, width);
+  FMS_REQUIRE(resid != nullptr && branch != nullptr, "norm_add_norm_affine: the stream and the branch are needed");
+  const bool vectors = branch_weight || branch_bias || weight || bias;
+  FMS_REQUIRE(!vectors || weight_dtype == FMS_F32 || weight_dtype == FMS_BF16, "norm_add_norm_affine: unknown weight dtype %d", weight_dtype);
+  const size_t lds = (size_t)width * sizeof(float);
+  if (act_dtype == FMS_F32)
+    norm_add_norm_affine_kernel<float><<<n_out, 256, lds, stream>>>(resid, (const float*)branch, branch_weight, branch_bias, branch_eps,
+                                                                    branch_mean, weight, bias, weight_dtype, eps, use_mean,
+                                                                    (float*)out, rows, width);
+  else if (act_dtype == FMS_BF16)
+    norm_add_norm_affine_kernel<bf16><<<n_out, 256, lds, stream>>>(resid, (const bf16*)branch, branch_weight, branch_bias, branch_eps,
+                                                                   branch_mean, weight, bias, weight_dtype, eps, use_mean,
+                                                                   (bf16*)out, rows, width);
+  else
+    FMS_REQUIRE(false, "norm_add_norm_affine: unknown dtype %d", act_dtype);
+  FMS_LAUNCH_CHECK("norm_add_norm_affine");
+  return 0;
+}

@@ -39,6 +39,9 @@ class StepBatch:
     # Rows of the logits that the caller asked for: the first n_wanted of the n_logit_rows that are computed (a
     # decode step padded to a row bucket computes a row for every padding token as well, as a captured step does).
     n_wanted: int = 0
+    # What a layer of this step leaves for later layers of the same step (tensors over the step's tokens, by name):
+    # emptied when a pass over the layers starts.
+    shared: Dict[str, torch.Tensor] = dataclasses.field(default_factory=dict)
 
 
 def build_batch(

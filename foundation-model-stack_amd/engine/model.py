@@ -131,6 +131,7 @@ class DecoderModel(Part):
     def forward(self, batch, cache: SequenceCache) -> torch.Tensor:
         """float32 logits [n wanted rows, vocab] of the tokens in `batch`; the cache is extended in place."""
         max_position = batch.max_context - 1
+        batch.shared.clear()
         stream = ResidualStream(self.embedding.forward(batch.token_ids, batch))
         for n, entry in enumerate(self.schedule):
             block = self.layers[entry.layer]

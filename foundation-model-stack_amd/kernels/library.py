@@ -17,7 +17,7 @@ import torch  # noqa: F401  (loads libamdhip64 before our library asks for it)
 
 from . import build as _build
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
@@ -33,9 +33,9 @@ _SIGNATURES = {
     "fmsamd_bias_add": [P, I, P, I, I, I, P],
     "fmsamd_rope_table": [P, P, P, I, I, P],
     "fmsamd_rope_kv_write": [P, I, L, P, P, P, I, P, P, I, I, P, P, I, I, I, I, I, P],
-    "fmsamd_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P, F, I, P],
-    "fmsamd_attn_prefill_bf16": [P, L, P, L, P, P, P, P, I, I, P, I, P, P, I, I, I, I, F, I, F, P],
-    "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, I, P, F, P],
+    "fmsamd_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P, F, I, I, I, P, P, I, P],
+    "fmsamd_attn_prefill_bf16": [P, L, P, L, P, P, P, P, I, I, P, I, P, P, I, I, I, I, F, I, F, I, P, P],
+    "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, I, P, F, I, P, P],
     "fmsamd_qkv_rope_skinny_bf16": [P, L, P, P, I, P, L, I, I, P, P, P, I, P, P, I, I, P, P, I, I, I, P, P, L, P],
     "fmsamd_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
     "fmsamd_gemm_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],
@@ -48,6 +48,7 @@ _SIGNATURES = {
     "fmsamd_sample": [P, L, I, I, I, F, I, P, P, P],
     "fmsamd_argmax": [P, L, I, I, P, L, P, P],
     "fmsamd_norm_add_norm": [P, P, I, P, F, P, I, F, P, P, I, I, P],
+    "fmsamd_norm_add_norm_affine": [P, P, I, P, P, F, I, P, P, I, F, I, P, P, I, I, P],
     "fmsamd_rms_norm_cols": [P, L, I, I, P, I, F, P, I, L, I, P],
     "fmsamd_activate": [P, P, I, L, I, P],
     "fmsamd_clamped_gated_act": [P, P, I, I, I, F, F, F, P],
@@ -67,8 +68,8 @@ _SIGNATURES = {
     "fmsamd_rglru_scan": [P, P, P, L, I, P, P, P, P, P, I, L, I, I, P],
     "fmsamd_rglru_scan_chunk": [I, I],
     "fmsamd_rglru_scan_chunked": [P, P, P, L, I, P, P, P, P, P, I, L, I, I, I, I, P, P],
-    "fmsamd_qk_projection_norm": [P, L, I, I, I, P, P, I, F, P, I, L, P, I, P],
-    "fmsamd_gate_mul": [P, L, P, L, I, F, P, L, I, I, I, P],
+    "fmsamd_qk_projection_norm": [P, L, I, I, I, P, P, I, F, P, I, L, P, I, I, P, L, P, P],
+    "fmsamd_gate_mul": [P, L, P, L, I, F, P, L, I, I, I, I, P],
     "fmsamd_scale_f32": [P, L, F, P],
     "fmsamd_cast_cols": [P, L, P, I, L, I, I, P],
     "fmsamd_delta_prepare": [P, L, I, P, L, I, P, I, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, P],

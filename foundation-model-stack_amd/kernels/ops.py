@@ -344,9 +344,20 @@ def attention(
     score_slopes: Optional[torch.Tensor] = None,
     soft_cap: float = 0.0,
     value_dim: int = 0,
+    chunk: int = 0,
+    keep_first: int = 0,
+    sink: Optional[torch.Tensor] = None,
+    distance_bias: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Causal attention of every token over the cache of its sequence -> [T, nheads*head_dim] (with value_dim, values
     and output heads of that size, through the generic kernel).
+
+    Which keys a query sees beside the causal rule: the last `window` (0: all), of which the sequence's first `keep_first`
+    keys are exempt; or, with chunk > 0 (and no window), the keys of the query's own run of `chunk` positions, counted from
+    the sequence's start.  sink: float32 [nheads], a logit per head that joins the softmax's denominator and has neither
+    key nor value.  distance_bias: float32 [nheads, L], added to the score by distance, min(distance, L - 1), neither
+    scaled nor capped.  The matrix-core kernels carry chunks and the sink; kept first keys and the distance bias run the
+    generic kernel in both types.
 
     Further terms of the scores (a position encoding that acts on the scores, a capped attention): score_slopes,
     float32 [nheads], adds slope[head] * (key position - query position); soft_cap c > 0 turns a score s into
@@ -373,14 +384,29 @@ def attention(
             raise ValueError(f"score_slopes must be a contiguous float32 [{nheads}] tensor")
     if not (soft_cap >= 0.0 and math.isfinite(soft_cap)):
         raise ValueError(f"soft_cap {soft_cap} must be zero (none) or positive")
+    chunk, keep_first = int(chunk), int(keep_first)
+    if chunk < 0 or keep_first < 0 or (chunk > 0 and (window > 0 or keep_first > 0)):
+        raise ValueError(f"chunks ({chunk}) go with neither a window ({window}) nor kept first keys ({keep_first}), and none is negative")
+    if sink is not None:
+        _need_cuda(sink)
+        if sink.dtype != torch.float32 or tuple(sink.shape) != (nheads,) or not sink.is_contiguous():
+            raise ValueError(f"sink must be a contiguous float32 [{nheads}] tensor")
+    dist_len = 0
+    if distance_bias is not None:
+        _need_cuda(distance_bias)
+        if distance_bias.dtype != torch.float32 or distance_bias.dim() != 2 or distance_bias.shape[0] != nheads or not distance_bias.is_contiguous():
+            raise ValueError(f"distance_bias must be a contiguous float32 [{nheads}, L] tensor")
+        dist_len = distance_bias.shape[1]
     if (q.dtype == torch.float32 or force_generic or head_dim % 16 or score_slopes is not None or value_dim
+            or keep_first or distance_bias is not None
             or (not decode and prefill_cap_is_generic(head_dim, soft_cap))):
         for t0 in range(0, T, 65535):
             n = min(65535, T - t0)
             check(lib.fmsamd_attn_generic(q[t0:].data_ptr(), q.stride(0), out[t0:].data_ptr(), out.stride(0), _code(q.dtype),
                                           positions[t0:].data_ptr(), seq_of_token[t0:].data_ptr(), block_table.data_ptr(),
                                           block_table.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), n, *common_tail[1:-1],
-                                          _ptr(score_slopes), float(soft_cap), value_dim, common_tail[-1]))
+                                          _ptr(score_slopes), float(soft_cap), value_dim, chunk, keep_first, _ptr(sink),
+                                          _ptr(distance_bias), dist_len, common_tail[-1]))
         return out
     if decode:
         if max_context <= 0:
@@ -404,7 +430,7 @@ def attention(
                                           block_table.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), T, nheads, kvheads,
                                           head_dim, float(scale), int(window), int(max_context), int(pages_per_block), int(waves),
                                           int(bool(staged)) if staged is not None else int(head_dim == 128), _ptr(row_order),
-                                          float(soft_cap), _stream()))
+                                          float(soft_cap), chunk, _ptr(sink), _stream()))
         return out
     if qblock_start is None or qblock_len is None:
         raise ValueError("bfloat16 prefill attention needs the query blocks of the batch")
@@ -413,7 +439,8 @@ def attention(
     check(lib.fmsamd_attn_prefill_bf16(q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), positions.data_ptr(),
                                        seq_of_token.data_ptr(), qblock_start.data_ptr(), qblock_len.data_ptr(),
                                        qblock_start.numel(), int(qblock_tokens), block_table.data_ptr(), block_table.stride(0),
-                                       k_cache.data_ptr(), v_cache.data_ptr(), *common_tail[:-1], float(soft_cap), common_tail[-1]))
+                                       k_cache.data_ptr(), v_cache.data_ptr(), *common_tail[:-1], float(soft_cap), chunk, _ptr(sink),
+                                       common_tail[-1]))
     return out
 
 
@@ -644,6 +671,53 @@ def norm_add_norm(
     check(load().fmsamd_norm_add_norm(resid.data_ptr(), branch.data_ptr(), _code(out_dtype), _ptr(branch_weight), float(branch_eps),
                                       _ptr(weight), _code(wdtype) if wdtype is not None else 0, float(eps), _ptr(out), _ptr(rows),
                                       n_out, width, _stream()))
+    return out
+
+
+def norm_add_norm_affine(
+    resid: torch.Tensor,
+    branch: torch.Tensor,
+    branch_weight: Optional[torch.Tensor],
+    branch_bias: Optional[torch.Tensor],
+    branch_eps: float,
+    branch_mean: bool,
+    weight: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    eps: float,
+    use_mean: bool,
+    out_dtype: torch.dtype,
+    rows: Optional[torch.Tensor] = None,
+    want_out: bool = True,
+) -> Optional[torch.Tensor]:
+    """norm_add_norm for norms that may take the mean off and add a shift: with N(v; w, b) = (v - mean) / sqrt(var + eps)
+    * w + b (var the mean of the squared deviations; without the mean flag no mean is taken off), resid += N(branch;
+    branch_weight, branch_bias) (float32, in place unless `rows` is given); returns N(resid; weight, bias) in `out_dtype`
+    (only `rows` if given; None if want_out is False)."""
+    _need_cuda(resid, branch, branch_weight, branch_bias, weight, bias, rows)
+    if resid.dtype != torch.float32 or resid.dim() != 2 or not resid.is_contiguous():
+        raise ValueError("the residual stream must be a contiguous float32 [T, width] tensor")
+    T, width = resid.shape
+    if branch.shape != resid.shape or not branch.is_contiguous() or branch.dtype != out_dtype:
+        raise ValueError(f"branch must be contiguous {tuple(resid.shape)} of {out_dtype}, got {tuple(branch.shape)} {branch.dtype}")
+    wdtype = None
+    for name, t in (("branch weight", branch_weight), ("branch bias", branch_bias), ("weight", weight), ("bias", bias)):
+        if t is not None:
+            if t.shape != (width,) or not t.is_contiguous():
+                raise ValueError(f"norm {name} must be a contiguous [{width}] tensor, got {tuple(t.shape)}")
+            if wdtype is not None and t.dtype != wdtype:
+                raise TypeError("the norms' weights and shifts must have one dtype")
+            wdtype = t.dtype
+    if width > 16384:
+        raise ValueError(f"norm_add_norm_affine keeps a row of at most 16384 elements, the width is {width}")
+    n_out = T
+    if rows is not None:
+        _need_i32("rows", rows)
+        n_out = rows.numel()
+    out = torch.empty(n_out, width, dtype=out_dtype, device=resid.device) if want_out else None
+    check(load().fmsamd_norm_add_norm_affine(resid.data_ptr(), branch.data_ptr(), _code(out_dtype), _ptr(branch_weight), _ptr(branch_bias),
+                                             float(branch_eps), int(bool(branch_mean)), _ptr(weight), _ptr(bias),
+                                             _code(wdtype) if wdtype is not None else 0, float(eps), int(bool(use_mean)), _ptr(out),
+                                             _ptr(rows), n_out, width, _stream()))
     return out
 
 
@@ -1100,15 +1174,28 @@ def moe_combine(y: torch.Tensor, weights: Optional[torch.Tensor], shared: Option
 # steps around attention
 # --------------------------------------------------------------------------
 def qk_projection_norm(proj: torch.Tensor, nq: int, nk: int, nv: int, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
-                       eps: float, out_dtype: torch.dtype, seq_of_token: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       eps: float, out_dtype: torch.dtype, seq_of_token: Optional[torch.Tensor] = None, norm_dim: int = 0,
+                       v_first: Optional[torch.Tensor] = None, v_lambda: Optional[torch.Tensor] = None) -> torch.Tensor:
     """float32 rows [q (nq) | k (nk) | v (nv) | ...] -> [T, nq + nk + nv] in out_dtype: q and k each RMS-normed over
-    their whole run of columns (all heads at once) times a weight, v as it is."""
-    _need_cuda(proj, q_weight, k_weight, seq_of_token)
+    their whole run of columns (all heads at once) times a weight, v as it is.  norm_dim > 0: the norms run over every
+    run of norm_dim columns (a head) by itself, with weights of norm_dim entries that all heads share.  v_first (rows
+    [T, nv] of out_dtype, any row stride) with v_lambda (one float32 number on the device): the values leave as
+    (1 - lambda) v + lambda v_first."""
+    _need_cuda(proj, q_weight, k_weight, seq_of_token, v_first, v_lambda)
+    norm_dim = int(norm_dim)
+    if norm_dim < 0 or (norm_dim and (nq % norm_dim or nk % norm_dim)):
+        raise ValueError(f"heads of {norm_dim} do not divide queries ({nq}) and keys ({nk})")
+    if v_first is not None:
+        _rows2d("v_first", v_first)
+        if v_first.dtype != out_dtype or tuple(v_first.shape) != (proj.shape[0], nv):
+            raise ValueError(f"v_first is [{proj.shape[0]}, {nv}] of {out_dtype}")
+        if v_lambda is None or v_lambda.dtype != torch.float32 or v_lambda.numel() != 1:
+            raise ValueError("blended values need their factor as one float32 number on the device")
     _rows2d("proj", proj)
     if proj.dtype != torch.float32 or proj.shape[1] < nq + nk + nv:
         raise ValueError("qk_projection_norm takes float32 rows that hold queries, keys and values")
     wdtype = None
-    for n, w in ((nq, q_weight), (nk, k_weight)):
+    for n, w in ((norm_dim or nq, q_weight), (norm_dim or nk, k_weight)):
         if w is not None:
             if tuple(w.shape) != (n,) or not w.is_contiguous() or (wdtype is not None and w.dtype != wdtype):
                 raise ValueError("the norm weights are contiguous vectors of the projections' sizes and of one type")
@@ -1118,28 +1205,33 @@ def qk_projection_norm(proj: torch.Tensor, nq: int, nk: int, nv: int, q_weight: 
     out = torch.empty(proj.shape[0], nq + nk + nv, dtype=out_dtype, device=proj.device)
     check(load().fmsamd_qk_projection_norm(proj.data_ptr(), proj.stride(0), nq, nk, nv, _ptr(q_weight), _ptr(k_weight),
                                            _code(wdtype) if wdtype is not None else 0, float(eps), out.data_ptr(), _code(out_dtype),
-                                           out.stride(0), _ptr(seq_of_token), proj.shape[0], _stream()))
+                                           out.stride(0), _ptr(seq_of_token), proj.shape[0], norm_dim, _ptr(v_first),
+                                           v_first.stride(0) if v_first is not None else 0, _ptr(v_lambda), _stream()))
     return out
 
 
 def gate_mul(x: torch.Tensor, gate: Optional[torch.Tensor], activation: str = "sigmoid", scale: float = 1.0,
-             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+             out: Optional[torch.Tensor] = None, group: int = 1) -> torch.Tensor:
     """x * act(gate) * scale, elementwise over rows [T, cols]; gate: float32 logits (a view with contiguous rows) or None;
-    out: rows of any stride to write into (default: a new tensor)."""
+    out: rows of any stride to write into (default: a new tensor).  group > 1: the gate has one column for every run of
+    `group` columns of x (a gate per head)."""
     _need_cuda(x, gate, out)
     _rows2d("x", x)
     T, cols = x.shape
+    group = int(group)
+    if group < 1 or cols % group:
+        raise ValueError(f"runs of {group} columns do not divide {cols}")
     if gate is not None:
         _rows2d("gate", gate)
-        if gate.dtype != torch.float32 or tuple(gate.shape) != (T, cols):
-            raise ValueError(f"the gate is float32 [{T}, {cols}]")
+        if gate.dtype != torch.float32 or tuple(gate.shape) != (T, cols // group):
+            raise ValueError(f"the gate is float32 [{T}, {cols // group}]")
     if out is None:
         out = torch.empty(T, cols, dtype=x.dtype, device=x.device)
     _rows2d("out", out)
     if out.dtype != x.dtype or tuple(out.shape) != (T, cols):
         raise ValueError(f"out is [{T}, {cols}] of the type of x")
     check(load().fmsamd_gate_mul(x.data_ptr(), x.stride(0), _ptr(gate), gate.stride(0) if gate is not None else 0, ACTIVATIONS[activation],
-                                 float(scale), out.data_ptr(), out.stride(0), _code(x.dtype), T, cols, _stream()))
+                                 float(scale), out.data_ptr(), out.stride(0), _code(x.dtype), T, cols, group, _stream()))
     return out
 
 

@@ -9,7 +9,7 @@ into steps changes nothing beyond rounding.
 
 Options, all constructor arguments: queries through a latent of their own with an RMS norm (q_rank; 0: the queries
 are one projection of the mixer's input), no rotated part at all (rot_dim 0, attention without positions), a sink logit
-per head in the softmax's denominator, a sigmoid gate per head on the output (read from the mixer's input), a
+per head in the softmax's denominator, a sigmoid gate per head or per output element (read from the mixer's input), a
 window, and `owns_kv=False` for a layer that reads the latent and key part that another layer cached (it then has
 no down-projection for them; its Uk, Uv, queries and everything else are its own).
 """
@@ -52,13 +52,16 @@ class LatentAttention(Mixer):
             raise ValueError("a rotated key part needs a position encoding")
         self.width, self.nheads, self.dim, self.rot_dim, self.vdim = width, nheads, dim, rot_dim, vdim
         self.q_rank, self.kv_rank, self.scale, self.eps = q_rank, kv_rank, float(scale), float(eps)
+        if output_gate not in (False, None, True, "head", "element"):
+            raise ValueError(f"output_gate {output_gate!r} is not one of False, True, 'head', 'element'")
         self.has_sink, self.has_gate, self.owns_kv, self.window = bool(sink), bool(output_gate), bool(owns_kv), int(window)
+        self.gate_cols = 0 if not output_gate else (nheads * vdim if output_gate == "element" else nheads)
         self.position_encoder = position_encoder
         # one product for everything that reads the mixer's input: [query latent (or the queries themselves) | gate logits |
         # kv latent, shared key part]
         self.q_cols = q_rank if q_rank else nheads * (dim + rot_dim)
         self.gate_col = self.q_cols
-        self.kv_col = self.q_cols + (nheads if output_gate else 0)
+        self.kv_col = self.q_cols + self.gate_cols
         self.down = self.add_child("down", Linear(width, self.kv_col + ((kv_rank + rot_dim) if owns_kv else 0)))
         if q_rank:
             self.declare("q_norm.weight", (q_rank,), init="ones", kind="scale")
@@ -78,7 +81,7 @@ class LatentAttention(Mixer):
         """The fused down-projection as the tensors it is made of, in the order of its rows (what the model's
         state_dict(fused_weights=False) shows in its place)."""
         H = self.nheads
-        pieces = [("dq" if self.q_rank else "q", self.q_cols)] + ([("g", H)] if self.has_gate else []) + ([("dkv", self.kv_rank + self.rot_dim)] if self.owns_kv else [])
+        pieces = [("dq" if self.q_rank else "q", self.q_cols)] + ([("g", self.gate_cols)] if self.has_gate else []) + ([("dkv", self.kv_rank + self.rot_dim)] if self.owns_kv else [])
         return {"down": tuple(pieces)}
 
     def kv_need(self) -> Optional[KVNeed]:
@@ -138,8 +141,12 @@ class LatentAttention(Mixer):
                                             self.scale, self.window, decode=batch.is_decode, max_context=batch.context_bound,
                                             vt_cache=cache.values)
         mixed = torch.empty(T, H * V, dtype=x.dtype, device=x.device)
-        gate = down[:, self.gate_col : self.gate_col + H] if self.has_gate else None
-        ops.headwise_linear(mixed_latent, R, self._uv, mixed, V, gate=gate)
+        gate = down[:, self.gate_col : self.gate_col + self.gate_cols] if self.has_gate else None
+        if self.gate_cols == H * V:  # a gate per output element: behind the product that leaves the latent space
+            ops.headwise_linear(mixed_latent, R, self._uv, mixed, V)
+            mixed = ops.gate_mul(mixed, gate, "sigmoid")
+        else:
+            ops.headwise_linear(mixed_latent, R, self._uv, mixed, V, gate=gate)
         return BranchOutput(mixed, self.o)
 
 

@@ -75,7 +75,12 @@ class ParameterizedNorm(Part):
                                         self.scale_weight(), self.groups, self.eps, rows)
         if branch_norm is not None and branch is not None:
             if not (self.deferrable() and branch_norm.deferrable()):
-                raise NotImplementedError("a normed branch is added by RMS norms without mean and shift only")
+                # norms that take the mean off or add a shift (layer norms): the general chain
+                vectors = [branch_norm.scale_weight(), branch_norm.w.get("bias"), self.scale_weight(), self.w.get("bias")]
+                if len({v.dtype for v in vectors if v is not None}) > 1:
+                    vectors = [v.to(torch.float32) if v is not None else None for v in vectors]  # the kernel takes one type
+                return ops.norm_add_norm_affine(resid, branch, vectors[0], vectors[1], branch_norm.eps, branch_norm.use_mean,
+                                                vectors[2], vectors[3], self.eps, self.use_mean, out_dtype, rows)
             return ops.norm_add_norm(resid, branch, branch_norm.scale_weight(), branch_norm.eps, self.scale_weight(), self.eps,
                                      out_dtype, rows)
         bias = self.w.get("bias")

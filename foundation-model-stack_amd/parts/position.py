@@ -39,6 +39,7 @@ def rope_frequencies(dim: int, theta: float, scaling: Optional[dict] = None, alp
 
     regular: fms/modules/positions.py:124-132.  llama3: fms/modules/positions.py:171-196.
     ntk: fms/modules/positions.py:161-168, theta * alpha^(dim / (dim - 2)) for the power of two `alpha`.
+    linear: every frequency divided by scaling["factor"].
     """
     scaling = dict(scaling or {})
     kind = scaling.get("rope_type", "regular")
@@ -52,6 +53,8 @@ def rope_frequencies(dim: int, theta: float, scaling: Optional[dict] = None, alp
         freqs = 1.0 / (theta ** (torch.arange(0, dim, 2)[: dim // 2].float() / dim))
     if kind in ("regular", "ntk"):
         return freqs.to(torch.float32)
+    if kind == "linear":  # positions counted in steps of 1 / factor: every frequency divided by the factor
+        return (freqs / float(scaling["factor"])).to(torch.float32)
     if kind == "llama3":
         factor = scaling["factor"]
         low_freq_factor = scaling["low_freq_factor"]
@@ -63,7 +66,7 @@ def rope_frequencies(dim: int, theta: float, scaling: Optional[dict] = None, alp
         smoothed = (1 - smooth) * scaled / factor + smooth * scaled
         medium = ~(wavelen < old_len / high_freq_factor) * ~(wavelen > old_len / low_freq_factor)
         return torch.where(medium, smoothed, scaled).to(torch.float32)
-    raise ValueError(f"rope_type {kind!r} is not supported (regular, llama3, ntk)")
+    raise ValueError(f"rope_type {kind!r} is not supported (regular, linear, llama3, ntk)")
 
 
 class PositionEncoding(Part):
