@@ -159,12 +159,13 @@ def attention_chunked(h, w, m, eps, state, positions):
     v = v.reshape(T, G, V)
     visible = visible_chunk(T, m["mask"]["size"])
     gate = torch.sigmoid(h @ w["g"].T)  # [T, H]
-    cap = m["softcap"]
+    cap = m.get("softcap")  # a configuration without one leaves the scores as they are
     out = torch.zeros(T, H, V, dtype=h.dtype)
     for head in range(H):
         g = head // (H // G)
         s = (q[:, head] @ k[:, g].T) * m["scale"]
-        s = cap * torch.tanh(s / cap)
+        if cap:
+            s = cap * torch.tanh(s / cap)
         p = _store(softmax_rows(s, visible, w["sink"][head]))
         out[:, head] = (p @ v[:, g]) * gate[:, head : head + 1]
     return _store(out.reshape(T, H * V)) @ w["o"].T + w["o.b"]
