@@ -128,6 +128,19 @@ __device__ __forceinline__ float capped(float raw, Scale2 s) {
   const float e = __builtin_amdgcn_exp2f(raw * (s.cap_in * 2.f * LOG2E));
   return __builtin_amdgcn_rcpf(s.cap_in) * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e));
 }
+// What the prompt kernels know beside window and chunk: the sequence's first `keep` keys stay visible in front of a window;
+// bias (or null): this head's row of a table by distance, bias[min(query position - key, len - 1)], added to the score as it
+// is (neither scaled nor capped: in units of the raw score it is bias / scale, hence inv_scale).
+struct ScoreExtras {
+  int keep;
+  const float* bias;
+  int len;
+  float inv_scale;
+};
+__device__ __forceinline__ float biased(float raw, int distance, const ScoreExtras& ex) {
+  const int n = distance < 0 ? 0 : (distance < ex.len ? distance : ex.len - 1);
+  return fmaf(ex.bias[n], ex.inv_scale, raw);
+}
 // the maximum that a partial result of the decode kernel carries when it holds no key at all
 #define DECODE_EMPTY -1e30f
 
@@ -218,7 +231,7 @@ __device__ __forceinline__ void step_scores(f32x4 (&sa)[QT], f32x4 (&sb)[QT], co
 template <int MAXDT, int QT>
 __device__ __forceinline__ void step_softmax(WaveState<MAXDT, QT>& st, f32x4 (&sa)[QT], f32x4 (&sb)[QT],
                                              bf16x8 (&pmat)[QT], const int (&qpos)[QT], const int (&qlo)[QT], int key0,
-                                             int head_dim, Scale2 scale2, bool full) {
+                                             int head_dim, Scale2 scale2, bool full, const ScoreExtras& ex) {
   const int g = (threadIdx.x & (WAVE - 1)) >> 4;
   const int ndt = head_dim / 16;
 #pragma unroll
@@ -229,13 +242,20 @@ __device__ __forceinline__ void step_softmax(WaveState<MAXDT, QT>& st, f32x4 (&s
 #pragma unroll
       for (int i = 0; i < 4; ++i) sa[qt][i] = capped(sa[qt][i], scale2), sb[qt][i] = capped(sb[qt][i], scale2);
     }
+    if (ex.bias != nullptr) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ja = key0 + g * 8 + i;
+        sa[qt][i] = biased(sa[qt][i], qpos[qt] - ja, ex), sb[qt][i] = biased(sb[qt][i], qpos[qt] - ja - 4, ex);
+      }
+    }
     if (!full) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int ja = key0 + g * 8 + i;  // the accumulator's rows 4 g + i hold these keys
         const int jb = ja + 4;
-        sa[qt][i] = (ja <= qpos[qt] && ja >= qlo[qt]) ? sa[qt][i] : -INFINITY;
-        sb[qt][i] = (jb <= qpos[qt] && jb >= qlo[qt]) ? sb[qt][i] : -INFINITY;
+        sa[qt][i] = (ja <= qpos[qt] && (ja >= qlo[qt] || ja < ex.keep)) ? sa[qt][i] : -INFINITY;
+        sb[qt][i] = (jb <= qpos[qt] && (jb >= qlo[qt] || jb < ex.keep)) ? sb[qt][i] : -INFINITY;
       }
     }
     float mx = max3f(max3f(sa[qt][0], sa[qt][1], sa[qt][2]), max3f(sa[qt][3], sb[qt][0], sb[qt][1]), max2f(sb[qt][2], sb[qt][3]));
@@ -285,11 +305,11 @@ template <int MAXDT, int QT>
 __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8 (&qreg)[QT][(MAXDT + 1) / 2],
                                           const int (&qpos)[QT], const int (&qlo)[QT], int key0, const bf16* kbase,
                                           int k_stride, const bf16* vbase, int v_stride, int head_dim, Scale2 scale2,
-                                          bool full) {
+                                          bool full, const ScoreExtras& ex = ScoreExtras{0, nullptr, 0, 0.f}) {
   f32x4 sa[QT], sb[QT];
   bf16x8 pmat[QT];
   step_scores<MAXDT, QT>(sa, sb, qreg, kbase, k_stride, head_dim);
-  step_softmax<MAXDT, QT>(st, sa, sb, pmat, qpos, qlo, key0, head_dim, scale2, full);
+  step_softmax<MAXDT, QT>(st, sa, sb, pmat, qpos, qlo, key0, head_dim, scale2, full, ex);
   step_accumulate<MAXDT, QT>(st, pmat, vbase, v_stride, head_dim);
 }
 
@@ -445,7 +465,7 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
                             int n_qblocks, const int* __restrict__ block_table, int table_stride,
                             const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, int nheads,
                             int kvheads, int head_dim_arg, float scale, int window, int hb, float soft_cap, int chunk,
-                            const float* __restrict__ sink) {
+                            const float* __restrict__ sink, int keep_first, const float* __restrict__ dist_bias, int dist_len) {
   const int head_dim = EXACT ? MAXDT * 16 : head_dim_arg;
   constexpr int KS = MAXDT * 16 + LDS_PAD;    // LDS row stride of the key page [64][KS]
   constexpr int VS = PAGE_TOKENS + LDS_PAD;   // LDS row stride of the transposed value page [head_dim][VS]
@@ -509,6 +529,16 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
   const int blk_hi = positions[t_end - 1];
   const int blk_lo = lower_bound(blk_first, window, chunk);
   const int page_first = blk_lo / PAGE_TOKENS, page_last = blk_hi / PAGE_TOKENS;
+  // The pages the block walks, counted through: first the pages of kept first keys that lie in front of the window, then
+  // page_first .. page_last.  walk_last is the last count; page_of turns a count into the sequence's page.
+  // (the kernel for head sizes between 64 and 128 has no register left for kept keys and the table either: the host sends
+  // such heads to the generic kernel)
+  if (MAXDT == 8 && !EXACT) keep_first = 0, dist_bias = nullptr;
+  const int kept_pages = (keep_first + PAGE_TOKENS - 1) / PAGE_TOKENS;
+  const int walk_kept = kept_pages < page_first ? kept_pages : page_first;
+  const int walk_last = walk_kept + page_last - page_first;
+  auto page_of = [&](int w) { return w < walk_kept ? w : page_first - walk_kept + w; };
+  const ScoreExtras ex = {keep_first, dist_bias != nullptr ? dist_bias + (size_t)h * dist_len : nullptr, dist_len, 1.f / scale};
 
   // cooperative copy: chunk id -> (row, 16-byte column) of the page in global memory and in LDS
   const int k_chunks = PAGE_TOKENS * head_dim / 8;  // per page; the value page has as many
@@ -547,26 +577,26 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
   // kbuf[i % PF], vbuf[i % PF]: page page_first + i on its way from memory.  The first page goes to LDS before
   // the loop; in the loop a page is multiplied while the next one is written to the other half of LDS and the
   // one PF further on is asked for: one barrier a page.
-  fetch(page_first, kbuf[0], vbuf[0]);
+  fetch(page_of(0), kbuf[0], vbuf[0]);
   stash(0, kbuf[0], vbuf[0]);
 #pragma unroll
-  for (int d = 0; d < PF; ++d) fetch(page_first + 1 + d <= page_last ? page_first + 1 + d : page_last, kbuf[(1 + d) % PF], vbuf[(1 + d) % PF]);
+  for (int d = 0; d < PF; ++d) fetch(page_of(1 + d <= walk_last ? 1 + d : walk_last), kbuf[(1 + d) % PF], vbuf[(1 + d) % PF]);
   block_sync_lds();  // not __syncthreads(): the pages under way must not be waited for
-  for (int p0 = page_first; p0 <= page_last; p0 += PF) {
+  for (int p0 = 0; p0 <= walk_last; p0 += PF) {
 #pragma unroll
     for (int d = 0; d < PF; ++d) {
       const int pi = p0 + d;  // past the last page (the loop runs in steps of PF pages): nothing but the barrier
       const int cur = d & 1;  // PF is even: the page's half of LDS
-      if (pi + 1 <= page_last) stash(cur ^ 1, kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
-      fetch(pi + 1 + PF <= page_last ? pi + 1 + PF : page_last, kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
-      const int key0 = pi * PAGE_TOKENS + khalf * 32;
-      if (has_work && pi <= page_last && !(key0 > wave_hi || key0 + 31 < wave_lo))  // uniform over the wave
+      if (pi + 1 <= walk_last) stash(cur ^ 1, kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
+      fetch(page_of(pi + 1 + PF <= walk_last ? pi + 1 + PF : walk_last), kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
+      const int key0 = page_of(pi) * PAGE_TOKENS + khalf * 32;
+      if (has_work && pi <= walk_last && key0 <= wave_hi && (key0 + 31 >= wave_lo || key0 < keep_first))  // uniform over the wave
         half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + cur * PAGE_ELEMS + khalf * 32 * KS, KS,
                              vs + cur * PAGE_ELEMS + khalf * 32, VS, head_dim,
                              // the kernel for head sizes between 64 and 128 has no register left for the cap (the host sends
                              // capped scores of such heads to the generic kernel)
                              make_scale2(scale, (MAXDT == 8 && !EXACT) ? 0.f : soft_cap),
-                             key0 + 31 <= full_hi && key0 >= full_lo);
+                             key0 + 31 <= full_hi && key0 >= full_lo, ex);
       block_sync_lds();  // the page just multiplied is overwritten after the next one
     }
   }
@@ -635,7 +665,7 @@ struct WaveState32 {
 template <int DT32>
 __device__ __forceinline__ void half_step32(WaveState32<DT32>& st, const bf16x8 (&qreg)[DT32 * 2], int qpos, int qlo,
                                             int key0, const bf16* kbase, int k_stride, const bf16* vbase, int v_stride,
-                                            Scale2 scale2, bool full) {
+                                            Scale2 scale2, bool full, const ScoreExtras& ex) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int j = lane & 31, hb = lane >> 5;
   // the key of tile row i = lane % 32 (this lane's row of the A operand): i = 8 blk + 4 h + e
@@ -654,11 +684,15 @@ __device__ __forceinline__ void half_step32(WaveState32<DT32>& st, const bf16x8 
 #pragma unroll
     for (int v = 0; v < 16; ++v) sc[v] = capped(sc[v], scale2);
   }
+  if (ex.bias != nullptr) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sc[v] = biased(sc[v], qpos - (key0 + 16 * (v >> 3) + 8 * hb + (v & 7)), ex);
+  }
   if (!full) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int key = key0 + 16 * (v >> 3) + 8 * hb + (v & 7);
-      sc[v] = (key <= qpos && key >= qlo) ? sc[v] : -INFINITY;
+      sc[v] = (key <= qpos && (key >= qlo || key < ex.keep)) ? sc[v] : -INFINITY;
     }
   }
   float mx = max3f(max3f(sc[0], sc[1], sc[2]), max3f(sc[3], sc[4], sc[5]), max3f(sc[6], sc[7], sc[8]));
@@ -705,7 +739,7 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
                               int n_qblocks, const int* __restrict__ block_table, int table_stride,
                               const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, int nheads,
                               int kvheads, float scale, int window, int hb, float soft_cap, int chunk,
-                              const float* __restrict__ sink) {
+                              const float* __restrict__ sink, int keep_first, const float* __restrict__ dist_bias, int dist_len) {
   constexpr int head_dim = DT32 * 32;
   constexpr int KS = head_dim + LDS_PAD;      // LDS row stride of the key page [64][KS]
   constexpr int VS = PAGE_TOKENS + LDS_PAD;   // LDS row stride of the transposed value page [head_dim][VS]
@@ -768,6 +802,13 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
   const int blk_hi = positions[t_end - 1];
   const int blk_lo = lower_bound(blk_first, window, chunk);
   const int page_first = blk_lo / PAGE_TOKENS, page_last = blk_hi / PAGE_TOKENS;
+  // The pages the block walks, counted through: first the pages of kept first keys that lie in front of the window, then
+  // page_first .. page_last.  walk_last is the last count; page_of turns a count into the sequence's page.
+  const int kept_pages = (keep_first + PAGE_TOKENS - 1) / PAGE_TOKENS;
+  const int walk_kept = kept_pages < page_first ? kept_pages : page_first;
+  const int walk_last = walk_kept + page_last - page_first;
+  auto page_of = [&](int w) { return w < walk_kept ? w : page_first - walk_kept + w; };
+  const ScoreExtras ex = {keep_first, dist_bias != nullptr ? dist_bias + (size_t)h * dist_len : nullptr, dist_len, 1.f / scale};
 
   constexpr int PF = 2;
   bf16x8 kbuf[PF][CH], vbuf[PF][CH];
@@ -801,22 +842,22 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
 #pragma unroll
     for (int v = 0; v < 16; ++v) st.acc[dt][v] = 0.f;
 
-  fetch(page_first, kbuf[0], vbuf[0]);
+  fetch(page_of(0), kbuf[0], vbuf[0]);
   stash(0, kbuf[0], vbuf[0]);
 #pragma unroll
-  for (int d = 0; d < PF; ++d) fetch(page_first + 1 + d <= page_last ? page_first + 1 + d : page_last, kbuf[(1 + d) % PF], vbuf[(1 + d) % PF]);
+  for (int d = 0; d < PF; ++d) fetch(page_of(1 + d <= walk_last ? 1 + d : walk_last), kbuf[(1 + d) % PF], vbuf[(1 + d) % PF]);
   block_sync_lds();  // not __syncthreads(): the pages under way must not be waited for
-  for (int p0 = page_first; p0 <= page_last; p0 += PF) {
+  for (int p0 = 0; p0 <= walk_last; p0 += PF) {
 #pragma unroll
     for (int d = 0; d < PF; ++d) {
       const int pi = p0 + d;  // past the last page (the loop runs in steps of PF pages): nothing but the barrier
       const int cur = d & 1;  // PF is even: the page's half of LDS
-      if (pi + 1 <= page_last) stash(cur ^ 1, kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
-      fetch(pi + 1 + PF <= page_last ? pi + 1 + PF : page_last, kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
-      const int key0 = pi * PAGE_TOKENS + khalf * 32;
-      if (has_work && pi <= page_last && !(key0 > wave_hi || key0 + 31 < wave_lo))  // uniform over the wave
+      if (pi + 1 <= walk_last) stash(cur ^ 1, kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
+      fetch(page_of(pi + 1 + PF <= walk_last ? pi + 1 + PF : walk_last), kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
+      const int key0 = page_of(pi) * PAGE_TOKENS + khalf * 32;
+      if (has_work && pi <= walk_last && key0 <= wave_hi && (key0 + 31 >= wave_lo || key0 < keep_first))  // uniform over the wave
         half_step32<DT32>(st, qreg, qpos, qlo, key0, ks + cur * PAGE_ELEMS + khalf * 32 * KS, KS,
-                          vs + cur * PAGE_ELEMS + khalf * 32, VS, make_scale2(scale, soft_cap), key0 + 31 <= full_hi && key0 >= full_lo);
+                          vs + cur * PAGE_ELEMS + khalf * 32, VS, make_scale2(scale, soft_cap), key0 + 31 <= full_hi && key0 >= full_lo, ex);
       block_sync_lds();  // the page just multiplied is overwritten after the next one
     }
   }
@@ -871,7 +912,8 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
 template <int MAXDT, int HALVES>
 __device__ __forceinline__ void decode_math(WaveState<MAXDT, 1>& st, const bf16x8 (&qreg)[(MAXDT + 1) / 2], int qpos,
                                             int qlo, int key0, const bf16x8 (&kreg)[HALVES][2][(MAXDT + 1) / 2],
-                                            const bf16x8 (&vreg)[HALVES][MAXDT], int head_dim, Scale2 scale2) {
+                                            const bf16x8 (&vreg)[HALVES][MAXDT], int head_dim, Scale2 scale2,
+                                            const ScoreExtras& ex) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int g = lane >> 4;
   const int ndt = head_dim / 16;
@@ -891,13 +933,17 @@ __device__ __forceinline__ void decode_math(WaveState<MAXDT, 1>& st, const bf16x
 #pragma unroll
       for (int i = 0; i < 4; ++i) sa[i] = capped(sa[i], scale2), sb[i] = capped(sb[i], scale2);
     }
+    if (ex.bias != nullptr) {  // this lane's column is a head of its own: its row of the table
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sa[i] = biased(sa[i], qpos - (k0 + g * 8 + i), ex), sb[i] = biased(sb[i], qpos - (k0 + g * 8 + i + 4), ex);
+    }
     if (!(k0 + 31 <= qpos && k0 >= qlo)) {  // uniform: not all 32 keys are visible
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int ja = k0 + g * 8 + i;  // the accumulator's rows 4 g + i hold these keys
         const int jb = ja + 4;
-        sa[i] = (ja <= qpos && ja >= qlo) ? sa[i] : -INFINITY;
-        sb[i] = (jb <= qpos && jb >= qlo) ? sb[i] : -INFINITY;
+        sa[i] = (ja <= qpos && (ja >= qlo || ja < ex.keep)) ? sa[i] : -INFINITY;
+        sb[i] = (jb <= qpos && (jb >= qlo || jb < ex.keep)) ? sb[i] : -INFINITY;
       }
     }
     float mx = max3f(max3f(sa[0], sa[1], sa[2]), max3f(sa[3], sb[0], sb[1]), max2f(sb[2], sb[3]));
@@ -930,7 +976,7 @@ __device__ __forceinline__ void decode_math(WaveState<MAXDT, 1>& st, const bf16x
 template <int MAXDT, int HALVES>
 __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x8 (&qreg)[(MAXDT + 1) / 2], int qpos,
                                             int qlo, int key0, const bf16* __restrict__ kp,
-                                            const bf16* __restrict__ vp, int head_dim, Scale2 scale2) {
+                                            const bf16* __restrict__ vp, int head_dim, Scale2 scale2, const ScoreExtras& ex) {
   // HALVES halves of 32 keys starting at key0 (kp/vp point at the page, `first` is the half inside it)
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
@@ -959,7 +1005,7 @@ __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x
     for (int dt = 0; dt < MAXDT; ++dt)
       vreg[hf][dt] = dt < ndt ? load_bf16x8(vp + (size_t)(dt * 16 + r) * PAGE_TOKENS + (first + hf) * 32 + g * 8) : zero8;
   }
-  decode_math<MAXDT, HALVES>(st, qreg, qpos, qlo, key0, kreg, vreg, head_dim, scale2);
+  decode_math<MAXDT, HALVES>(st, qreg, qpos, qlo, key0, kreg, vreg, head_dim, scale2, ex);
 }
 
 // Pages of head size 128 by way of the wave's own 16 KB of LDS.  The page of a kv head is 16 KB of keys and
@@ -985,7 +1031,8 @@ __device__ __forceinline__ void staged_load(bf16x8 (&raw)[16], const bf16* __res
 template <bool PREFETCH>
 __device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16x8 (&qreg)[4], int qpos, int qlo,
                                                  int key0, bf16x8 (&raw)[16], const bf16* __restrict__ vp,
-                                                 const bf16* __restrict__ kn, bf16* __restrict__ buf, Scale2 scale2) {
+                                                 const bf16* __restrict__ kn, bf16* __restrict__ buf, Scale2 scale2,
+                                                 const ScoreExtras& ex) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
   const int g = lane >> 4;
@@ -1028,6 +1075,15 @@ __device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16
 #pragma unroll
       for (int i = 0; i < 4; ++i) sa[hf][i] = capped(sa[hf][i], scale2), sb[hf][i] = capped(sb[hf][i], scale2);
   }
+  if (ex.bias != nullptr) {  // this lane's column is a head of its own: its row of the table
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ja = key0 + hf * 32 + g * 8 + i;
+        sa[hf][i] = biased(sa[hf][i], qpos - ja, ex), sb[hf][i] = biased(sb[hf][i], qpos - ja - 4, ex);
+      }
+  }
   if (!(key0 + PAGE_TOKENS - 1 <= qpos && key0 >= qlo)) {  // uniform: not all 64 keys are visible
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf)
@@ -1035,8 +1091,8 @@ __device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16
       for (int i = 0; i < 4; ++i) {
         const int ja = key0 + hf * 32 + g * 8 + i;  // the accumulator's rows 4 g + i hold these keys
         const int jb = ja + 4;
-        sa[hf][i] = (ja <= qpos && ja >= qlo) ? sa[hf][i] : -INFINITY;
-        sb[hf][i] = (jb <= qpos && jb >= qlo) ? sb[hf][i] : -INFINITY;
+        sa[hf][i] = (ja <= qpos && (ja >= qlo || ja < ex.keep)) ? sa[hf][i] : -INFINITY;
+        sb[hf][i] = (jb <= qpos && (jb >= qlo || jb < ex.keep)) ? sb[hf][i] : -INFINITY;
       }
   }
   float mx = -INFINITY;
@@ -1093,36 +1149,50 @@ __device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16
   __builtin_amdgcn_wave_barrier();  // the values have been read: the buffer is free for the next page's keys
 }
 
-// The pages first, first + stride, ... <= last of a sequence, for kv head kh.
+// A sequence's pages as a query walks them, counted through: first the walk.kept pages of kept first keys that lie in front
+// of the window, then the pages from walk.first on.
+struct PageWalk {
+  int kept, first;
+  __device__ __forceinline__ int page(int w) const { return w < kept ? w : first - kept + w; }
+};
+
+// The pages of the counts first, first + stride, ... <= last of a sequence's walk, for kv head kh.
 __device__ __forceinline__ void decode_pages_staged(WaveState<8, 1>& st, const bf16x8 (&qreg)[4], int qpos, int qlo,
-                                                    int first, int stride, int last, const int* __restrict__ bt,
+                                                    int first, int stride, int last, PageWalk walk, const int* __restrict__ bt,
                                                     const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
-                                                    size_t page_elems, int kh, bf16* __restrict__ buf, Scale2 scale2) {
+                                                    size_t page_elems, int kh, bf16* __restrict__ buf, Scale2 scale2,
+                                                    const ScoreExtras& ex) {
   if (first > last) return;
   const size_t head_off = (size_t)kh * PAGE_TOKENS * 128;
   bf16x8 raw[16];
-  size_t phys = readable_page(uniform_load(bt + first));
+  size_t phys = readable_page(uniform_load(bt + walk.page(first)));
   staged_load(raw, k_cache + phys * page_elems + head_off);
   int pi = first;
   for (; pi + stride <= last; pi += stride) {
-    const size_t next = readable_page(uniform_load(bt + pi + stride));
-    staged_page_step<true>(st, qreg, qpos, qlo, pi * PAGE_TOKENS, raw, v_cache + phys * page_elems + head_off,
-                           k_cache + next * page_elems + head_off, buf, scale2);
+    const size_t next = readable_page(uniform_load(bt + walk.page(pi + stride)));
+    staged_page_step<true>(st, qreg, qpos, qlo, walk.page(pi) * PAGE_TOKENS, raw, v_cache + phys * page_elems + head_off,
+                           k_cache + next * page_elems + head_off, buf, scale2, ex);
     phys = next;
   }
-  staged_page_step<false>(st, qreg, qpos, qlo, pi * PAGE_TOKENS, raw, v_cache + phys * page_elems + head_off, nullptr,
-                          buf, scale2);
+  staged_page_step<false>(st, qreg, qpos, qlo, walk.page(pi) * PAGE_TOKENS, raw, v_cache + phys * page_elems + head_off, nullptr,
+                          buf, scale2, ex);
 }
 
 // The pages that split `split` of `n_splits` takes of a sequence whose visible keys are lo..pos: every
 // sequence's own pages are dealt out evenly, so that in a batch of unequal lengths every block has work in
 // proportion to its sequence.  Returns the number of splits that have pages at all (the first ones).
-__device__ __forceinline__ int split_pages(int lo, int pos, int n_splits, int split, int* page_lo, int* page_hi) {
+// (with kept first keys the pages in front of the window are dealt out with the others: page_lo and page_hi are counts of
+// the walk, which walk.page() turns into pages)
+__device__ __forceinline__ int split_pages(int lo, int pos, int keep, int n_splits, int split, PageWalk* walk, int* page_lo,
+                                           int* page_hi) {
   const int first_page = lo / PAGE_TOKENS, last_page = pos / PAGE_TOKENS;
-  const int span = last_page - first_page + 1;
+  const int kept_pages = (keep + PAGE_TOKENS - 1) / PAGE_TOKENS;
+  walk->kept = kept_pages < first_page ? kept_pages : first_page;
+  walk->first = first_page;
+  const int span = walk->kept + last_page - first_page + 1;
   const int per = (span + n_splits - 1) / n_splits;
-  *page_lo = first_page + split * per;
-  *page_hi = *page_lo + per - 1 < last_page ? *page_lo + per - 1 : last_page;
+  *page_lo = split * per;
+  *page_hi = *page_lo + per - 1 < span - 1 ? *page_lo + per - 1 : span - 1;
   return (span + per - 1) / per;
 }
 
@@ -1139,7 +1209,7 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
                             const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                             const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
                             int window, int tile_cols, const int* __restrict__ row_order, float soft_cap, int chunk,
-                            const float* __restrict__ sink) {
+                            const float* __restrict__ sink, int keep_first, const float* __restrict__ dist_bias, int dist_len) {
   extern __shared__ float lds_dynamic[];  // not staged: [wave][tile_cols columns][head_dim + 2]
   __shared__ __attribute__((aligned(16))) bf16 stage[STAGED ? MAXW * 8192 : 8];
   // where the waves' partial results meet: a region of its own, or (staged) the head of each wave's page buffer
@@ -1178,8 +1248,12 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
   }
   const int pos = uniform_load(positions + t);
   const int lo = lower_bound(pos, window, chunk);
+  // (the kernel that stages pages of head size 128 in LDS has no register left for kept keys and the table: the host
+  // sends such steps to the kernel that loads straight into registers)
+  if (STAGED) keep_first = 0, dist_bias = nullptr;
   int page_lo, page_hi;
-  if (split >= split_pages(lo, pos, n_splits, split, &page_lo, &page_hi)) {
+  PageWalk walk;
+  if (split >= split_pages(lo, pos, keep_first, n_splits, split, &walk, &page_lo, &page_hi)) {
     leave_empty();
     return;
   }
@@ -1192,20 +1266,24 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
 
   WaveState<MAXDT, 1> st;
   wave_state_init(st);
+  // a lane's column is a query head: its row of the distance table
+  const ScoreExtras ex = {keep_first, dist_bias != nullptr ? dist_bias + (size_t)(head0 + (r < cols ? r : 0)) * dist_len : nullptr,
+                          dist_len, 1.f / scale};
   if (STAGED) {
     if constexpr (MAXDT == 8)
-      decode_pages_staged(st, qreg, pos, lo, page_lo + wave, n_waves, page_hi, bt, k_cache, v_cache, page_elems, kh,
-                          stage + wave * 8192, make_scale2(scale, soft_cap));
+      decode_pages_staged(st, qreg, pos, lo, page_lo + wave, n_waves, page_hi, walk, bt, k_cache, v_cache, page_elems, kh,
+                          stage + wave * 8192, make_scale2(scale, soft_cap), ex);
   } else {
-    for (int pi = page_lo + wave; pi <= page_hi; pi += n_waves) {
+    for (int wi = page_lo + wave; wi <= page_hi; wi += n_waves) {
+      const int pi = walk.page(wi);
       const size_t phys = readable_page(uniform_load(bt + pi));
       const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
       const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
       if (MAXDT <= 8) {
-        decode_keys<MAXDT, 2>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, make_scale2(scale, soft_cap));
+        decode_keys<MAXDT, 2>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, make_scale2(scale, soft_cap), ex);
       } else {  // large heads: half a page at a time keeps the loads in registers
-        decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, make_scale2(scale, soft_cap));
-        decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS + 32, kp, vp, head_dim, make_scale2(scale, soft_cap));
+        decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, make_scale2(scale, soft_cap), ex);
+        decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS + 32, kp, vp, head_dim, make_scale2(scale, soft_cap), ex);
       }
     }
   }
@@ -1384,8 +1462,12 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
                                         const int* block_table, int table_stride, const void* k_cache,
                                         const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
                                         float scale, int window, float soft_cap, int chunk, const float* sink,
-                                        hipStream_t stream) {
+                                        int keep_first, const float* dist_bias, int dist_len, hipStream_t stream) {
   if (n_tokens == 0 || n_qblocks == 0) return 0;
+  FMS_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attn_prefill_bf16: kept first keys (%d) go with a window", keep_first);
+  FMS_REQUIRE(dist_bias == nullptr || dist_len > 0, "attn_prefill_bf16: a distance table needs a length");
+  FMS_REQUIRE((head_dim <= 64 || head_dim == 128) || (keep_first == 0 && dist_bias == nullptr),
+              "attn_prefill_bf16: kept first keys and a distance table of head size %d go through attn_generic", head_dim);
   FMS_REQUIRE(chunk >= 0 && !(chunk > 0 && window > 0), "attn_prefill_bf16: a window (%d) and chunks (%d) do not go together", window, chunk);
   if (check_common("attn_prefill_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_prefill_bf16: head size %d is no multiple of 16", head_dim);
@@ -1417,17 +1499,17 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
     attn_prefill_lds_kernel<M, LDS_QT, LDS_UNITS, true><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(          \
         (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,       \
         n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads,         \
-        head_dim, scale, window, hb, soft_cap, chunk, sink);                                                       \
+        head_dim, scale, window, hb, soft_cap, chunk, sink, keep_first, dist_bias, dist_len);                      \
   else                                                                                                             \
     attn_prefill_lds_kernel<M, LDS_QT, LDS_UNITS, false><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(         \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,         \
       n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, \
-      scale, window, hb, soft_cap, chunk, sink);                                                                   \
+      scale, window, hb, soft_cap, chunk, sink, keep_first, dist_bias, dist_len);                                  \
   } while (0)
 #define FMS_PL32(D32)                                                                                              \
   attn_prefill_lds32_kernel<D32, LDS_UNITS><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(                      \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len, n_qblocks, \
-      block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, scale, window, hb, soft_cap, chunk, sink)
+      block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, scale, window, hb, soft_cap, chunk, sink, keep_first, dist_bias, dist_len)
   if (head_dim == 128)  // head sizes with a 32x32x16 kernel of their own
     FMS_PL32(4);
   else if (head_dim == 64)
@@ -1453,8 +1535,10 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
                                        const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
                                        float scale, int window, int max_context, int pages_per_split, int waves,
                                        int staged, const int* row_order, float soft_cap, int chunk, const float* sink,
-                                       hipStream_t stream) {
+                                       int keep_first, const float* dist_bias, int dist_len, hipStream_t stream) {
   if (n_tokens == 0) return 0;
+  FMS_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attn_decode_bf16: kept first keys (%d) go with a window", keep_first);
+  FMS_REQUIRE(dist_bias == nullptr || dist_len > 0, "attn_decode_bf16: a distance table needs a length");
   FMS_REQUIRE(chunk >= 0 && !(chunk > 0 && window > 0), "attn_decode_bf16: a window (%d) and chunks (%d) do not go together", window, chunk);
   if (check_common("attn_decode_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_decode_bf16: head size %d is no multiple of 16", head_dim);
@@ -1481,8 +1565,9 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
   attn_decode_bf16_kernel<M, MAXW, STAGED><<<grid, dim3(waves * WAVE), LDS, stream>>>(                               \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, part_o, part_ml, n_splits, positions, seq_of_token,          \
       block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale,       \
-      window, tile_cols, row_order, soft_cap, chunk, sink)
+      window, tile_cols, row_order, soft_cap, chunk, sink, keep_first, dist_bias, dist_len)
   FMS_REQUIRE(staged == 0 || head_dim == 128, "attn_decode_bf16: pages go through LDS for head size 128 only");
+  FMS_REQUIRE(staged == 0 || (keep_first == 0 && dist_bias == nullptr), "attn_decode_bf16: kept first keys and a distance table go with pages loaded straight into registers (staged = 0)");
   if (staged != 0) {
     // the waves' results meet in the page buffers: 16 KB a wave hold 16 columns of 130 floats
     if (waves <= 4)

@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define FMSAMD_ABI_VERSION 8
+#define FMSAMD_ABI_VERSION 10
 
 // element types
 #define FMS_F32 0
@@ -76,7 +76,7 @@ int fmsamd_attn_generic(const void* q, long q_stride, void* out, long out_stride
                         const float* sink, const float* dist_bias, int dist_len, hipStream_t stream);
 
 // soft_cap (0: none) of the two bfloat16 kernels: scores become soft_cap * tanh(score / soft_cap); chunk and sink as in
-// fmsamd_attn_generic.
+// fmsamd_attn_generic; so are keep_first and dist_bias (the prefill kernel has them for head sizes up to 64, and for 128).
 // bfloat16 prefill: the step is cut into query blocks of at most fmsamd_attn_prefill_qblock(...) consecutive
 // tokens of one sequence; the same number goes into the call as qblock_tokens
 int fmsamd_attn_prefill_qblock(int nheads, int kvheads, int head_dim, int n_tokens);
@@ -84,7 +84,8 @@ int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_s
                              const int* seq_of_token, const int* qblock_start, const int* qblock_len, int n_qblocks,
                              int qblock_tokens, const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
                              int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
-                             float soft_cap, int chunk, const float* sink, hipStream_t stream);
+                             float soft_cap, int chunk, const float* sink, int keep_first, const float* dist_bias,
+                             int dist_len, hipStream_t stream);
 
 // bfloat16 decode: one token per sequence.  The context bound max_context is cut into splits of
 // `pages_per_split` pages, and every sequence deals its own pages out evenly over that many blocks of `waves`
@@ -98,7 +99,8 @@ int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, long out_st
                             const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
                             int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
                             int max_context, int pages_per_split, int waves, int staged, const int* row_order,
-                            float soft_cap, int chunk, const float* sink, hipStream_t stream);
+                            float soft_cap, int chunk, const float* sink, int keep_first, const float* dist_bias,
+                            int dist_len, hipStream_t stream);
 
 // c[M, N] = a[M, K] w[N, K]^T (+ bias[N])
 int fmsamd_gemm_f32(const float* a, long lda, const float* w, const float* bias, float* c, long ldc, int M, int N,

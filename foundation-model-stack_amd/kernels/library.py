@@ -17,7 +17,7 @@ import torch  # noqa: F401  (loads libamdhip64 before our library asks for it)
 
 from . import build as _build
 
-ABI_VERSION = 8
+ABI_VERSION = 10
 
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
@@ -34,8 +34,8 @@ _SIGNATURES = {
     "fmsamd_rope_table": [P, P, P, I, I, P],
     "fmsamd_rope_kv_write": [P, I, L, P, P, P, I, P, P, I, I, P, P, I, I, I, I, I, P],
     "fmsamd_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P, F, I, I, I, P, P, I, P],
-    "fmsamd_attn_prefill_bf16": [P, L, P, L, P, P, P, P, I, I, P, I, P, P, I, I, I, I, F, I, F, I, P, P],
-    "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, I, P, F, I, P, P],
+    "fmsamd_attn_prefill_bf16": [P, L, P, L, P, P, P, P, I, I, P, I, P, P, I, I, I, I, F, I, F, I, P, I, P, I, P],
+    "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, I, P, F, I, P, I, P, I, P],
     "fmsamd_qkv_rope_skinny_bf16": [P, L, P, P, I, P, L, I, I, P, P, P, I, P, P, I, I, P, P, I, I, I, P, P, L, P],
     "fmsamd_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
     "fmsamd_gemm_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],

@@ -356,8 +356,8 @@ def attention(
     keys are exempt; or, with chunk > 0 (and no window), the keys of the query's own run of `chunk` positions, counted from
     the sequence's start.  sink: float32 [nheads], a logit per head that joins the softmax's denominator and has neither
     key nor value.  distance_bias: float32 [nheads, L], added to the score by distance, min(distance, L - 1), neither
-    scaled nor capped.  The matrix-core kernels carry chunks and the sink; kept first keys and the distance bias run the
-    generic kernel in both types.
+    scaled nor capped.  The matrix-core kernels carry chunks and the sink; kept first keys and the distance bias the
+    matrix-core decode kernel, and the matrix-core prompt kernel for head sizes up to 64 and for 128.
 
     Further terms of the scores (a position encoding that acts on the scores, a capped attention): score_slopes,
     float32 [nheads], adds slope[head] * (key position - query position); soft_cap c > 0 turns a score s into
@@ -397,8 +397,9 @@ def attention(
         if distance_bias.dtype != torch.float32 or distance_bias.dim() != 2 or distance_bias.shape[0] != nheads or not distance_bias.is_contiguous():
             raise ValueError(f"distance_bias must be a contiguous float32 [{nheads}, L] tensor")
         dist_len = distance_bias.shape[1]
+    prefill_extras = bool(keep_first) or distance_bias is not None  # kept keys or a table: not every matrix-core kernel has them
     if (q.dtype == torch.float32 or force_generic or head_dim % 16 or score_slopes is not None or value_dim
-            or keep_first or distance_bias is not None
+            or (prefill_extras and not decode and (prefill_extras_are_generic(head_dim) or qblock_start is None))
             or (not decode and prefill_cap_is_generic(head_dim, soft_cap))):
         for t0 in range(0, T, 65535):
             n = min(65535, T - t0)
@@ -429,8 +430,8 @@ def attention(
                                           positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
                                           block_table.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), T, nheads, kvheads,
                                           head_dim, float(scale), int(window), int(max_context), int(pages_per_block), int(waves),
-                                          int(bool(staged)) if staged is not None else int(head_dim == 128), _ptr(row_order),
-                                          float(soft_cap), chunk, _ptr(sink), _stream()))
+                                          int(bool(staged)) if staged is not None else int(head_dim == 128 and not prefill_extras), _ptr(row_order),
+                                          float(soft_cap), chunk, _ptr(sink), keep_first, _ptr(distance_bias), dist_len, _stream()))
         return out
     if qblock_start is None or qblock_len is None:
         raise ValueError("bfloat16 prefill attention needs the query blocks of the batch")
@@ -440,7 +441,7 @@ def attention(
                                        seq_of_token.data_ptr(), qblock_start.data_ptr(), qblock_len.data_ptr(),
                                        qblock_start.numel(), int(qblock_tokens), block_table.data_ptr(), block_table.stride(0),
                                        k_cache.data_ptr(), v_cache.data_ptr(), *common_tail[:-1], float(soft_cap), chunk, _ptr(sink),
-                                       common_tail[-1]))
+                                       keep_first, _ptr(distance_bias), dist_len, common_tail[-1]))
     return out
 
 
@@ -464,6 +465,12 @@ def prefill_cap_is_generic(head_dim: int, soft_cap: float) -> bool:
     """True if capped scores of this head size run the generic kernel in multi-token steps: the matrix-core prefill
     kernel for head sizes between 64 and 128 has no cap."""
     return soft_cap > 0.0 and 64 < head_dim < 128
+
+
+def prefill_extras_are_generic(head_dim: int) -> bool:
+    """True if kept first keys and a distance table of this head size run the generic kernel in multi-token steps: the
+    matrix-core prefill kernels carry them for head sizes up to 64 and for 128."""
+    return head_dim > 64 and head_dim != 128
 
 
 def prefill_qblock(nheads: int, kvheads: int, head_dim: int, n_tokens: int) -> int:

@@ -184,7 +184,8 @@ class MultiHeadAttention(Mixer):
 
     def prefill_qblock(self, n_tokens: int, dtype) -> int:
         if (dtype != torch.bfloat16 or self.head_dim % 16 or self._score_slopes() is not None or self.value_dim != self.head_dim
-                or self.keep_first or self.distance_bias is not None or ops.prefill_cap_is_generic(self.head_dim, self.soft_cap)):
+                or ((self.keep_first or self.distance_bias is not None) and ops.prefill_extras_are_generic(self.head_dim))
+                or ops.prefill_cap_is_generic(self.head_dim, self.soft_cap)):
             return 0  # the generic kernel takes tokens one by one
         return ops.prefill_qblock(self.nheads, self.kvheads, self.head_dim, n_tokens)
 

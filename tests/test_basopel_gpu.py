@@ -317,6 +317,11 @@ MASKS = [
     (8, 1, 32, 32, 0, 0, 150, 10.0, False, None),         # ... without a sink,
     (2, 2, 96, 96, 0, 0, 7, 12.0, True, None),            # ... a head size between 64 and 128
     (2, 1, 128, 128, 50, 0, 0, 20.0, True, None),         # a window and a sink
+    (4, 2, 128, 128, 70, 5, 0, 0.0, False, (32, 64)),     # kept keys and a distance table on the matrix-core prompt kernels:
+    (4, 1, 64, 64, 40, 130, 0, 0.0, True, (16, 200)),     # ... three pages of kept keys, a table longer than the window,
+    (2, 2, 32, 32, 100, 64, 0, 9.0, False, (8, 20)),      # ... a page of kept keys exactly, a cap,
+    (3, 3, 80, 80, 30, 1, 0, 0.0, False, (6, 9)),         # ... a head size without a kernel of its own
+    (2, 2, 48, 48, 64, 2, 0, 0.0, False, None),           # ... kept keys without a table
 ]
 
 
@@ -373,7 +378,7 @@ def test_attention_masks_sink_and_distance_bias(lib, dtype, sizes):
         common = dict(soft_cap=cap, value_dim=V, chunk=chunk, keep_first=keep, sink=sink.to(DEV) if has_sink else None, distance_bias=by_distance)
         # as a prompt
         qb = {}
-        if dtype == torch.bfloat16 and D == V and D % 16 == 0 and not keep and table is None and not ops.prefill_cap_is_generic(D, cap):
+        if dtype == torch.bfloat16 and D == V and D % 16 == 0 and (not ops.prefill_extras_are_generic(D) or (not keep and table is None)) and not ops.prefill_cap_is_generic(D, cap):
             size = ops.prefill_qblock(H, K, D, n)
             starts = list(range(0, n, size))
             qb = dict(qblock_start=torch.tensor(starts, dtype=torch.int32, device=DEV),
