@@ -23,6 +23,12 @@ flops would take at what this GPU delivers (`x_roofline`: 1 is the roofline).
 is the same comparison for Defapel (windowed attention beside a gated delta rule, a delta rule with a decay per channel,
 experts weighted on their input) beside Llama of the same width, depth and heads.
 
+    python bench.py --basopel [--layers N]
+
+is the same comparison for Basopel (attention in chunks with a sink, in a window that keeps first tokens with a bias by
+distance, and over a latent; layer norms on both sides of every branch) beside Llama of the same width, depth, heads and
+gated feed-forward; every attention call is priced by the keys its own mask shows.
+
     python bench.py --sidalorn [--layers N]
 
 is the same comparison for Sidalorn (attention without positions over a latent, a real-gated recurrent block, norms in

@@ -412,6 +412,15 @@ def attention(
     if decode:
         if max_context <= 0:
             raise ValueError("decode attention needs max_context (an upper bound of every context length)")
+        # a window or a chunk bounds the pages a query can see whatever its context: the step is cut for that many, so
+        # that long contexts do not launch splits that find no key
+        seen = 0
+        if window > 0:
+            seen = -(-int(window) // PAGE_TOKENS) + 1 + -(-keep_first // PAGE_TOKENS)
+        elif chunk > 0:
+            seen = -(-chunk // PAGE_TOKENS) + 1
+        if seen:
+            max_context = min(int(max_context), seen * PAGE_TOKENS)
         n_pages = -(-max_context // PAGE_TOKENS)
         auto_pages, auto_waves = decode_split(T * kvheads, n_pages)
         if pages_per_block <= 0:
