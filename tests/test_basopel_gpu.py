@@ -597,6 +597,71 @@ def test_the_edges_decide_in_prompts_and_in_decoding(lib, name, tmp_path):
                 judge(run(250), want, "float32")
 
 
+def drawn_configuration(seed):
+    """A configuration whose every size, count, constant and layer order is drawn at random (the layers that mix values
+    agree in key/value heads times value size, as they must)."""
+    import random
+
+    rng = random.Random(seed)
+    mixed = rng.choice([48, 96])  # key/value heads times value size of the layers that mix their values
+    layers = []
+    for _ in range(rng.randint(2, 5)):
+        kind = rng.choice(["c", "c", "w", "l"])
+        ff = rng.choice([None, 24, 50, 64, 128])
+        if kind == "l":
+            rot = rng.choice([2, 4, 8, 16, 32])
+            layers.append(layer(latent(rng.randint(1, 4), rng.choice([8, 12, 16, 32, 64]), rot, rng.choice([8, 20, 32, 64]),
+                                       rng.choice([8, 16, 24, 64]), rng.randint(1, 150), base=rng.choice([10.0, 1e4, 5e5]),
+                                       scale=rng.uniform(0.1, 0.4)), ff))
+            continue
+        v_mix = rng.random() < 0.7
+        if v_mix:
+            kv = rng.choice([g for g in (1, 2, 3, 4, 6) if mixed % g == 0])
+            vdim = mixed // kv
+        else:
+            kv, vdim = rng.choice([1, 2, 3]), rng.choice([8, 16, 40, 64])
+        heads = kv * rng.choice([1, 2, 4])
+        dim = rng.choice([8, 16, 20, 32, 48, 64, 96, 128]) if rng.random() < 0.7 else vdim + vdim % 2
+        if kind == "c":
+            dims = rng.choice([d for d in (2, 4, 8, 16, 32, 48, 64, 128) if d <= dim])
+            layers.append(layer(chunked(heads, kv, dim, vdim, rng.randint(1, 180), dims, base=rng.choice([100.0, 1e4, 2.5e5]),
+                                        factor=rng.choice([None, 2.0, 8.0]), scale=rng.uniform(0.1, 0.4), softcap=rng.choice([None, 5.0, 20.0, 50.0]),
+                                        v_mix=v_mix), ff))
+        else:
+            rows = rng.choice([2, 4, 8, 16, 32])
+            layers.append(layer(windowed(heads, kv, dim, vdim, rng.randint(1, 180), rng.choice([None, 0, 1, 4, 70]), rows,
+                                         rng.randint(rows // 2 + 1, 200), scale=rng.uniform(0.1, 0.4), v_mix=v_mix), ff))
+    return dict(vocab=rng.randint(50, 600), width=rng.choice([64, 96, 100, 128, 192]), norm={"eps": rng.choice([1e-6, 1e-5, 1e-3])},
+                embedding={"scale": rng.uniform(0.5, 12.0)}, max_positions=1024, layers=layers)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_configurations_drawn_at_random(lib, seed, tmp_path):
+    """Every size, constant and layer order drawn: whole, in portions and token by token in float32; whole in bfloat16."""
+    from fms_amd.engine import Engine
+
+    folder = write_folder(lib, str(tmp_path / "drawn"), drawn_configuration(seed), seed=100 + seed)
+    cfg, weights = P.load_model_folder(folder)
+    ids = tokens_for(cfg["vocab"], 200, seed)
+    for dtype in DTYPES:
+        want = expect(cfg, weights, ids, dtype)
+        model = lib.get_model("hf_pretrained", model_path=folder, data_type=dtype)
+        engine = Engine(model, max_tokens=256, max_slots=1)
+        slot = engine.new_sequence()
+        judge(engine.step([slot], [ids], "all"), want, dtype)
+        engine.end_sequence(slot)
+        if dtype == "float32":
+            for cuts in ([70, 1, 2, 127], [130] + [1] * 70):
+                slot = engine.new_sequence()
+                got, at = [], 0
+                for n in cuts:
+                    got.append(engine.step([slot], [ids[at : at + n]], "all"))
+                    at += n
+                judge(torch.cat(got), want, dtype)
+                engine.end_sequence(slot)
+        engine.cache.check()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding_through_graphs_and_eager_steps(lib, folders, dtype):
     """300 tokens decoded one by one for three sequences of different lengths, across page borders, past windows and
